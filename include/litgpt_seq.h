@@ -44,6 +44,16 @@ int lgs_linear(const void* a, long lda, long stride_a, const void* w, int w_f32,
 /* x[t] = table[tokens[t]] * scale */
 int lgs_embed(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W, int vocab,
               lgs_stream_t stream);
+/* x[t] = table[tokens[t]] * scale + pos_table[pos[t]] (both tables of one dtype); x_bf16: optional rounded copy */
+int lgs_embed_pos(const int* tokens, const int* pos, const void* table, const void* pos_table, int w_f32, float scale,
+                  float* x, void* x_bf16, int T, int W, int vocab, int positions, lgs_stream_t stream);
+/* layer norm of a sublayer's output y [rows][n] joining the residual x [rows][n]:
+ * x (+)= mult * ((y - mean) / sqrt(var + eps) * weight + bias), var = mean of the squared deviations (bias may be
+ * NULL; accumulate 0 writes instead of adding); x_bf16: optional copy of the new x rounded to bf16 */
+int lgs_layernorm(const float* y, const float* weight, const float* bias, float eps, float mult, int accumulate,
+                  float* x, void* x_bf16, int rows, int n, lgs_stream_t stream);
+/* z[i] = cap * tanh(z[i] / cap) in place */
+int lgs_softcap(float* z, long n, float cap, lgs_stream_t stream);
 /* group g of row r: y = x / sqrt(mean(x^2) + eps) * (offset + weight) (weight NULL: unit RMS), n values per group */
 int lgs_rmsnorm(const float* x, long ldx, const float* weight, float offset, float eps, float* y, long ldy, int rows,
                 int groups, int n, void* y_bf16 /* optional rounded copy, same layout */, lgs_stream_t stream);
@@ -61,9 +71,11 @@ int lgs_retention(float* q, float* k, const float* v, long ld, float* state, con
                   const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
                   int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked, float* ws, int max_chunks,
                   int T_rows, const int* pos, lgs_stream_t stream);
-/* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * act(g[t * ldg + h * dv + i]) */
+/* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * weight[i] * act(g[t * ldg + h * dv + i]) * post
+ * (weight: dv values shared by the heads, or NULL) */
 int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps, int act,
-                  void* o_bf16 /* optional rounded copy [T][H * dv] */, lgs_stream_t stream);
+                  const float* weight, float post, void* o_bf16 /* optional rounded copy [T][H * dv] */,
+                  lgs_stream_t stream);
 /* latent attention, per token: c = rmsnorm(proj[kv_off .. + r]) * norm_w -> cache_c[slot][pos] (bf16, or fp32 with
  * cache_f32); rotary (pairs 2i, 2i + 1) of proj[kv_off + r .. + dr] -> cache_kr[slot][pos] (fp32); the rotated
  * part of every head's query (at q_off + h (d + dr) + d) is rotated in place. */
@@ -91,19 +103,27 @@ int lgs_glu(const float* a, const float* b, long ld, void* out /* fp32, or bf16 
 /* per token: ids / wts [T][top] = the top largest of z[t * ld .. + E] (lowest index first among equals) and the
  * softmax over those. E <= 256. */
 int lgs_moe_route(const float* z, long ld, int T, int E, int top, int* ids, float* wts, lgs_stream_t stream);
-/* streaming experts: actbuf[t * top + k] = act(up[ids[t][k]] h[t]); x[t] += sum_k wts[t][k] down[ids[t][k]] actbuf[..] */
+/* per token: s = softmax(z[t * ld .. + E]) over all E outputs; ids = the top largest of s + bias (bias NULL: of s;
+ * lowest index first among equals), wts = s at those places (not renormalised). E <= 256. */
+int lgs_moe_route_scores(const float* z, long ld, int T, int E, int top, const float* bias, int* ids, float* wts,
+                         lgs_stream_t stream);
+/* streaming experts: actbuf[t * top + k] = act(up[ids[t][k]] h[t]), or with gated (up holds per expert F gate rows,
+ * then F up rows) act(gate h) * (up h); x[t] (+)= sum_k wts[t][k] down[ids[t][k]] actbuf[..]. An id >= n_real names
+ * an identity expert without matrices: it is skipped by lgs_moe_up and contributes wts * hin[t] in lgs_moe_down. */
 int lgs_moe_up(const float* h, long ldh, const void* up, int w_f32, const int* ids, float* actbuf, int T, int top,
-               int F, int K, int act, lgs_stream_t stream);
+               int F, int K, int act, int gated, int n_real, lgs_stream_t stream);
 int lgs_moe_down(const float* actbuf, const void* down, int w_f32, const int* ids, const float* wts, float* x,
-                 long ldx, int T, int top, int N, int F, lgs_stream_t stream);
+                 long ldx, int T, int top, int N, int F, int n_real, const float* hin, long ldh, int accumulate,
+                 lgs_stream_t stream);
 /* counting sort of the (token, choice) pairs by expert: z_start [E + 1], tok_of [pairs] (token of each sorted entry),
  * where [pairs] (sorted place of each pair); the order inside an expert's range is not fixed. ws: 2 E ints, zero on
  * entry, left zero. */
 int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where, int* ws,
                  lgs_stream_t stream);
-/* x[t] += sum_k wts[t][k] * y[where[t * top + k]] */
+/* x[t] (+)= sum_k wts[t][k] * y[where[t * top + k]]; with ids, a choice with ids[t][k] >= n_real (an identity expert)
+ * contributes hin[t] instead of a row of y */
 int lgs_moe_combine(const float* y, const int* where, const float* wts, float* x, long ldx, int T, int top, int N,
-                    lgs_stream_t stream);
+                    const int* ids, int n_real, const float* hin, long ldh, int accumulate, lgs_stream_t stream);
 /* x[t] += unit_rms(proj_w (gelu_tanh(gate_w x[t]) * table[tokens[t]][col0 .. + dim])) * norm_w */
 int lgs_token_side(float* x, const int* tokens, const void* table, int w_f32, long ld_table, int col0,
                    const void* gate_w, const void* proj_w, const float* norm_w, int T, int W, int dim, int vocab,
@@ -138,6 +158,38 @@ int lgs_diffattn(const float* q, long ld, const void* cache_k, const void* cache
                  const int* seq_slot, const int* seq_pos0, float* out, void* out_bf16, float* part, int splits, int B,
                  int max_len, int H, int G, int d, int dv, int max_seq, int chunk, float scale, float cap, float lambda,
                  float eps, float post, lgs_stream_t stream);
+
+/* ---- softmax attention with unit-RMS queries and keys and a sink ---- */
+/* Per token: every query head at proj[q_off ..] is divided by its root mean square (eps inside the root) and
+ * multiplied by the query temperature 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: 1),
+ * in place; every key head at proj[k_off ..] is divided by its root mean square on its way to cache_k
+ * [slots][max_seq][G][d]; the values at proj[v_off ..] go to cache_v [slots][max_seq][G][dv] (bf16, or fp32). */
+int lgs_normattn_prepare(float* proj, long ld, int q_off, int k_off, int v_off, void* cache_k, void* cache_v,
+                         int cache_f32, const int* slot, const int* pos, int T, int H, int G, int d, int dv, int max_seq,
+                         float eps, float temp_coef, int temp_every, lgs_stream_t stream);
+/* out[t][h] = post * sum_j p_j v_j over the cached rows j of the mask (as lgs_diffattn's), p = softmax of
+ * cap((q . k_j) * scale) with exp(sink[h]) added to the normaliser (sink NULL: none); grouped key / value heads.
+ * One map per head: q rows hold d values per head. max_len, splits and part (T H splits (2 + dv) floats) as in
+ * lgs_diffattn. */
+int lgs_sinkattn(const float* q, long ld, const void* cache_k, const void* cache_v, int cache_f32, const float* sink,
+                 const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, void* out_bf16, float* part,
+                 int splits, int B, int max_len, int H, int G, int d, int dv, int max_seq, int chunk, float scale,
+                 float cap, float post, lgs_stream_t stream);
+
+/* ---- gated delta rule ---- */
+/* Per token, on rows qkv [T][ld] = q [G][d] | k [G][d] | v [H][dv] (after their convolution): q and k become unit
+ * vectors per head, x / sqrt(sum(x^2) + norm_eps), q also times q_scale, in place; beta[t][h] = sigmoid(b[t ldb + h]);
+ * dec = exp(-exp(A_log[h]) softplus(a + dt_bias)) with a, dt_bias and dec per head and key channel ([H][d],
+ * per_channel) or per head ([H]). */
+int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb, const float* A_log,
+                      const float* dt_bias, float* dec, float* beta, int T, int H, int G, int d, int per_channel,
+                      float q_scale, float norm_eps, lgs_stream_t stream);
+/* Per sequence and head, token by token: S <- diag(dec) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.
+ * Head h reads q / k head h / (H / G). state [slots][H][d][dv] fp32 is read unless the sequence starts at position 0
+ * and written back. d <= 512. lanes: lanes that share a state column (4, 8 or 16; 0: chosen from the sizes). */
+int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, float* state, const int* seq_start,
+                    const int* seq_slot, const int* seq_pos0, float* out, int B, int H, int G, int d, int dv,
+                    int per_channel, int lanes, lgs_stream_t stream);
 
 /* ---- selective state-space mixer ---- */
 /* out[t][c] = silu(bias[c] + sum_j w[c][j] u[t - (taps - 1 - j)][c]) per sequence of a packed batch; inputs before

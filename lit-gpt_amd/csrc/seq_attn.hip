@@ -76,27 +76,66 @@ __global__ void __launch_bounds__(256) diffattn_prepare_kernel(AttnPrepArgs p) {
   }
 }
 
+struct NormPrepArgs {
+  float* proj;
+  long ld;
+  int q_off, k_off, v_off;
+  void* cache_k;  // [slots][S][G][d]
+  void* cache_v;  // [slots][S][G][dv]
+  const int *slot, *pos;
+  int H, G, d, dv, S, temp_every;
+  float eps, temp_coef;
+};
+
+// grid (T): wave w takes the vectors w, w + 4, ... of the H query heads (divided by their root mean square and
+// multiplied by the position's query temperature, in place) and of the G key heads (divided by their root mean
+// square on their way into the cache); then all threads copy the values into the cache.
+template <bool CF32>
+__global__ void __launch_bounds__(256) normattn_prepare_kernel(NormPrepArgs p) {
+  const size_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = p.pos[t], d = p.d;
+  float* row = p.proj + t * p.ld;
+  const size_t crow = ((size_t)p.slot[t] * p.S + pos) * p.G;
+  const float temp = p.temp_every > 0 ? 1.0f + p.temp_coef * logf((float)((pos + 1) / p.temp_every + 1)) : 1.0f;
+  for (int vec = wave; vec < p.H + p.G; vec += 4) {
+    const bool isk = vec >= p.H;
+    float* x = row + (isk ? p.k_off + (size_t)(vec - p.H) * d : p.q_off + (size_t)vec * d);
+    float ss = 0.0f;
+    for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
+    ss = wave_sum(ss);
+    const float s = (isk ? 1.0f : temp) / sqrtf(ss / (float)d + p.eps);
+    for (int i = lane; i < d; i += 64) {
+      if (isk) cstore<CF32>(p.cache_k, (crow + (vec - p.H)) * d + i, x[i] * s);
+      else x[i] *= s;
+    }
+  }
+  const int nv = p.G * p.dv;
+  for (int i = threadIdx.x; i < nv; i += 256) cstore<CF32>(p.cache_v, crow * p.dv + i, row[p.v_off + i]);
+}
+
 struct AttnArgs {
-  const float* q;  // rotated queries at q + row * ld + h * 2 d
+  const float* q;  // prepared queries at q + row * ld + h * MAPS d
   long ld;
   const void* cache_k;
   const void* cache_v;
   const int *seq_start, *seq_slot, *seq_pos0;
   float* out;       // [T][H * dv]
   uint16_t* out16;  // optional bf16 copy
-  float* part;      // splits > 1: [T][H][splits][4 + 2 dv]
+  float* part;      // splits > 1: [T][H][splits][MAPS (2 + dv)]
   int H, G, d, dv, S, chunk, tiles;
   float scale, cap, lambda, eps, post;
+  const float* sink;  // one map: exp(sink[h]) joins the softmax normaliser (NULL: no sink)
 };
 
 constexpr int kKeyTile = 256;
 // row stride of the score / weight tile in LDS, [key][(query, map)]: a key's weights for all queries and maps lie
 // side by side, so the value phase fetches them with 16-byte reads
-template <int QT>
-constexpr int score_stride() { return QT == 1 ? 4 : 2 * QT + 4; }
+template <int NR>
+constexpr int score_stride() { return NR <= 2 ? 4 : NR + 4; }
 
-// o = a1 / l1 - lambda a2 / l2 over the head, unit RMS, times post. Called by all 256 threads; thread c < dv owns
-// column c (dv <= 256).
+// two maps: o = a1 / l1 - lambda a2 / l2 over the head, unit RMS, times post. Called by all 256 threads; thread
+// c < dv owns column c (dv <= 256).
 __device__ __forceinline__ void diff_finish(float a1, float a2, float l1, float l2, const AttnArgs& p, size_t row, int h,
                                             float* red) {
   const int c = threadIdx.x;
@@ -110,19 +149,39 @@ __device__ __forceinline__ void diff_finish(float a1, float a2, float l1, float 
   }
 }
 
-// grid (B * tiles, H, splits). LDS: queries [QT][2 d], scores / weights [256][2 QT + 4], per (query, map) the running
+// one map: o = a / (l + exp(sink - m)) times post, with a and l relative to the running maximum m
+__device__ __forceinline__ void sink_finish(float a, float m, float l, const AttnArgs& p, size_t row, int h) {
+  const int c = threadIdx.x;
+  float den = l, num = a;
+  if (p.sink) {
+    const float s = p.sink[h], top = fmaxf(m, s);
+    const float w = m == -INFINITY ? 0.0f : expf(m - top);
+    den = l * w + expf(s - top);
+    num = a * w;
+  }
+  if (c < p.dv) {
+    const float v = num / den * p.post;
+    const size_t at = row * p.H * p.dv + (size_t)h * p.dv + c;
+    p.out[at] = v;
+    if (p.out16) p.out16[at] = f2bf(v);
+  }
+}
+
+// grid (B * tiles, H, splits). MAPS maps per head (2: differential attention, 1: plain softmax attention with an
+// optional sink). LDS: queries [QT][MAPS d], scores / weights [256][QT MAPS + 4], per (query, map) the running
 // maximum, normaliser and the rescale of the current tile, and the cross-subset sums of the value phase.
-template <int QT, bool CF32>
+template <int QT, int MAPS, bool CF32>
 __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
   extern __shared__ float lds[];
   __shared__ float red[4];
-  const int d = p.d, dv = p.dv, d2 = 2 * d;
+  constexpr int NR = QT * MAPS;  // (query, map) rows
+  const int d = p.d, dv = p.dv, d2 = MAPS * d;
   float* qs = lds;                       // [QT][d2]
-  constexpr int SCS = score_stride<QT>();
+  constexpr int SCS = score_stride<NR>();
   float* sc = qs + QT * d2;              // [kKeyTile][SCS]: scores, then weights, of key x (query, map)
-  float* mrow = sc + kKeyTile * SCS;     // [2 QT] running maximum
-  float* lrow = mrow + 2 * QT;           // [2 QT] running normaliser
-  float* arow = lrow + 2 * QT;           // [2 QT] rescale of what was summed before this tile
+  float* mrow = sc + kKeyTile * SCS;     // [NR] running maximum
+  float* lrow = mrow + NR;               // [NR] running normaliser
+  float* arow = lrow + NR;               // [NR] rescale of what was summed before this tile
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int b = blockIdx.x / p.tiles, tile = blockIdx.x % p.tiles;
   const int h = blockIdx.y, g = h / (p.H / p.G);
@@ -140,7 +199,7 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
     hi = min(hi, lo + per);
   }
   for (int i = tid; i < nq * d2; i += 256) qs[i] = p.q[(size_t)(r0 + i / d2) * p.ld + (size_t)h * d2 + i % d2];
-  if (tid < 2 * QT) {
+  if (tid < NR) {
     mrow[tid] = -INFINITY;
     lrow[tid] = 0.0f;
   }
@@ -148,22 +207,27 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
   int ncol = 64;
   while (ncol < dv) ncol <<= 1;  // dv <= 256
   const int KS = 256 / ncol, col = tid % ncol, ks = tid / ncol;
-  float acc[QT][2];
+  float acc[QT][MAPS];
 #pragma unroll
-  for (int i = 0; i < QT; ++i) acc[i][0] = acc[i][1] = 0.0f;
+  for (int i = 0; i < QT; ++i)
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) acc[i][m] = 0.0f;
   __syncthreads();
 
   for (int k0 = lo; k0 < hi; k0 += kKeyTile) {
     const int nk = min(kKeyTile, hi - k0);
     // ---- scores of key k0 + tid against every query and map
     {
-      float s[QT][2];
+      float s[QT][MAPS];
 #pragma unroll
-      for (int i = 0; i < QT; ++i) s[i][0] = s[i][1] = 0.0f;
+      for (int i = 0; i < QT; ++i)
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) s[i][m] = 0.0f;
       if (tid < nk) {
         const size_t kr = ((slot * p.S + k0 + tid) * p.G + g) * d2;
         if ((d & 3) == 0) {
-          for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m)
             for (int e = 0; e < d; e += 4) {
               float kv[4];
               if (CF32) {
@@ -183,7 +247,8 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
               }
             }
         } else {
-          for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m)
             for (int e = 0; e < d; ++e) {
               const float kv = cload<CF32>(p.cache_k, kr + m * d + e);
 #pragma unroll
@@ -198,16 +263,16 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
         const int qlo = chunk > 0 ? qpos - qpos % chunk : 0;
         const bool see = tid < nk && i < nq && kpos <= qpos && kpos >= qlo;
 #pragma unroll
-        for (int m = 0; m < 2; ++m) {
+        for (int m = 0; m < MAPS; ++m) {
           float v = s[i][m] * p.scale;
           if (p.cap > 0.0f) v = p.cap * tanhf(v / p.cap);
-          sc[tid * SCS + 2 * i + m] = see ? v : -INFINITY;
+          sc[tid * SCS + MAPS * i + m] = see ? v : -INFINITY;
         }
       }
     }
     __syncthreads();
-    // ---- online softmax: wave w owns rows w, w + 4, ... of the 2 QT (query, map) rows
-    for (int r = wave; r < 2 * QT; r += 4) {
+    // ---- online softmax: wave w owns rows w, w + 4, ... of the (query, map) rows
+    for (int r = wave; r < NR; r += 4) {
       float* srow = sc + r;
       float v[4], mx = -INFINITY;
 #pragma unroll
@@ -236,102 +301,110 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
     // ---- weighted sums of the values
     {
 #pragma unroll
-      for (int i = 0; i < QT; ++i) {
-        acc[i][0] *= arow[2 * i];
-        acc[i][1] *= arow[2 * i + 1];
-      }
+      for (int i = 0; i < QT; ++i)
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) acc[i][m] *= arow[MAPS * i + m];
       if (col < dv) {
 #pragma unroll 4
         for (int j = ks; j < nk; j += KS) {
           const float v = cload<CF32>(p.cache_v, ((slot * p.S + k0 + j) * p.G + g) * dv + col);
-          float w[2 * QT];
-          if (QT == 1) {
+          float w[NR];
+          if (NR == 1) {
+            w[0] = sc[j * SCS];
+          } else if (NR == 2) {
             const float2 t = *(const float2*)(sc + j * SCS);
-            w[0] = t.x, w[1] = t.y;
+            w[0] = t.x, w[NR - 1] = t.y;
           } else {
 #pragma unroll
-            for (int e = 0; e < 2 * QT; e += 4) {
+            for (int e = 0; e + 3 < NR; e += 4) {
               const float4 t = *(const float4*)(sc + j * SCS + e);
               w[e] = t.x, w[e + 1] = t.y, w[e + 2] = t.z, w[e + 3] = t.w;
             }
           }
 #pragma unroll
-          for (int i = 0; i < QT; ++i) {
-            acc[i][0] = fmaf(w[2 * i], v, acc[i][0]);
-            acc[i][1] = fmaf(w[2 * i + 1], v, acc[i][1]);
-          }
+          for (int i = 0; i < QT; ++i)
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m) acc[i][m] = fmaf(w[MAPS * i + m], v, acc[i][m]);
         }
       }
     }
     __syncthreads();
   }
   // ---- sum the key subsets (fixed order), then finish or leave the split's partial result
-  float* xs = sc;  // [KS][2 QT][ncol] = 256 * 2 QT floats <= the score tile
+  float* xs = sc;  // [KS][NR][ncol] = 256 * NR floats <= the score tile
   if (KS > 1) {
 #pragma unroll
-    for (int i = 0; i < QT; ++i) {
-      xs[(ks * 2 * QT + 2 * i) * ncol + col] = acc[i][0];
-      xs[(ks * 2 * QT + 2 * i + 1) * ncol + col] = acc[i][1];
-    }
+    for (int i = 0; i < QT; ++i)
+#pragma unroll
+      for (int m = 0; m < MAPS; ++m) xs[(ks * NR + MAPS * i + m) * ncol + col] = acc[i][m];
     __syncthreads();
   }
   for (int i = 0; i < nq; ++i) {
-    float a1 = 0.0f, a2 = 0.0f;
+    float a[MAPS];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) a[m] = 0.0f;
     if (KS > 1) {
       if (tid < ncol)
-        for (int z = 0; z < KS; ++z) {
-          a1 += xs[(z * 2 * QT + 2 * i) * ncol + tid];
-          a2 += xs[(z * 2 * QT + 2 * i + 1) * ncol + tid];
-        }
+        for (int z = 0; z < KS; ++z)
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m) a[m] += xs[(z * NR + MAPS * i + m) * ncol + tid];
     } else {
 #pragma unroll
       for (int e = 0; e < QT; ++e)  // (static indexing keeps acc in registers)
-        if (e == i) a1 = acc[e][0], a2 = acc[e][1];
+        if (e == i)
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m) a[m] = acc[e][m];
     }
     if (gridDim.z > 1) {
-      float* pr = p.part + (((size_t)(r0 + i) * p.H + h) * gridDim.z + blockIdx.z) * (4 + 2 * dv);
-      if (tid == 0) pr[0] = mrow[0], pr[1] = lrow[0], pr[2] = mrow[1], pr[3] = lrow[1];
-      if (tid < dv) pr[4 + tid] = a1, pr[4 + dv + tid] = a2;
+      float* pr = p.part + (((size_t)(r0 + i) * p.H + h) * gridDim.z + blockIdx.z) * (MAPS * (2 + dv));
+      if (tid < MAPS) pr[2 * tid] = mrow[tid], pr[2 * tid + 1] = lrow[tid];
+      if (tid < dv)
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) pr[2 * MAPS + m * dv + tid] = a[m];
+    } else if (MAPS == 2) {
+      diff_finish(a[0], a[MAPS - 1], lrow[MAPS * i], lrow[MAPS * i + MAPS - 1], p, (size_t)(r0 + i), h, red);
     } else {
-      diff_finish(a1, a2, lrow[2 * i], lrow[2 * i + 1], p, (size_t)(r0 + i), h, red);
+      sink_finish(a[0], mrow[i], lrow[i], p, (size_t)(r0 + i), h);
     }
   }
 }
 
 // grid (T, H): merges the splits of one (token, head) in split order and finishes
+template <int MAPS>
 __global__ void __launch_bounds__(256) diffattn_combine_kernel(AttnArgs p, int splits) {
   __shared__ float red[4];
   const size_t t = blockIdx.x;
   const int h = blockIdx.y, dv = p.dv, c = threadIdx.x;
-  const float* pr = p.part + ((t * p.H + h) * splits) * (4 + 2 * dv);
-  float m1 = -INFINITY, m2 = -INFINITY;
+  const int stride = MAPS * (2 + dv);
+  const float* pr = p.part + ((t * p.H + h) * splits) * stride;
+  float mx[MAPS], l[MAPS], a[MAPS];
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) mx[m] = -INFINITY, l[m] = 0.0f, a[m] = 0.0f;
+  for (int z = 0; z < splits; ++z)
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) mx[m] = fmaxf(mx[m], pr[(size_t)z * stride + 2 * m]);
   for (int z = 0; z < splits; ++z) {
-    m1 = fmaxf(m1, pr[(size_t)z * (4 + 2 * dv)]);
-    m2 = fmaxf(m2, pr[(size_t)z * (4 + 2 * dv) + 2]);
-  }
-  float l1 = 0.0f, l2 = 0.0f, a1 = 0.0f, a2 = 0.0f;
-  for (int z = 0; z < splits; ++z) {
-    const float* q = pr + (size_t)z * (4 + 2 * dv);
-    const float w1 = q[0] == -INFINITY ? 0.0f : expf(q[0] - m1), w2 = q[2] == -INFINITY ? 0.0f : expf(q[2] - m2);
-    l1 = fmaf(q[1], w1, l1);
-    l2 = fmaf(q[3], w2, l2);
-    if (c < dv) {
-      a1 = fmaf(q[4 + c], w1, a1);
-      a2 = fmaf(q[4 + dv + c], w2, a2);
+    const float* q = pr + (size_t)z * stride;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      const float w = q[2 * m] == -INFINITY ? 0.0f : expf(q[2 * m] - mx[m]);
+      l[m] = fmaf(q[2 * m + 1], w, l[m]);
+      if (c < dv) a[m] = fmaf(q[2 * MAPS + m * dv + c], w, a[m]);
     }
   }
-  diff_finish(a1, a2, l1, l2, p, t, h, red);
+  if (MAPS == 2) diff_finish(a[0], a[MAPS - 1], l[0], l[MAPS - 1], p, t, h, red);
+  else sink_finish(a[0], mx[0], l[0], p, t, h);
 }
 
-template <int QT>
+template <int QT, int MAPS>
 static size_t diffattn_lds(int d) {
-  return sizeof(float) * ((size_t)QT * 2 * d + (size_t)kKeyTile * score_stride<QT>() + 6 * QT);
+  return sizeof(float) * ((size_t)QT * MAPS * d + (size_t)kKeyTile * score_stride<QT * MAPS>() + 3 * QT * MAPS);
 }
 
-template <int QT>
+template <int QT, int MAPS>
 static int diffattn_launch(const AttnArgs& p, int cache_f32, dim3 grid, hipStream_t stream) {
-  const size_t lds = diffattn_lds<QT>(p.d);
-  auto* fn = cache_f32 ? diffattn_kernel<QT, true> : diffattn_kernel<QT, false>;
+  const size_t lds = diffattn_lds<QT, MAPS>(p.d);
+  auto* fn = cache_f32 ? diffattn_kernel<QT, MAPS, true> : diffattn_kernel<QT, MAPS, false>;
   if (lds > 48 * 1024) {
     const hipError_t e = hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
@@ -374,16 +447,57 @@ extern "C" int lgs_diffattn(const float* q, long ld, const void* cache_k, const 
   LGA_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || (part && max_len == 1)),
                 "lgs_diffattn: splits need one token per sequence and a workspace");
   lgs::AttnArgs p{q, ld, cache_k, cache_v, seq_start, seq_slot, seq_pos0, out, (uint16_t*)out_bf16, part,
-                  H, G, d, dv, max_seq, chunk, 0, scale, cap, lambda, eps, post};
+                  H, G, d, dv, max_seq, chunk, 0, scale, cap, lambda, eps, post, nullptr};
   int rc;
   if (max_len == 1) {
     p.tiles = 1;
-    rc = lgs::diffattn_launch<1>(p, cache_f32, dim3(B, H, splits), stream);
-    if (rc == 0 && splits > 1) lgs::diffattn_combine_kernel<<<dim3(B, H), 256, 0, stream>>>(p, splits);
+    rc = lgs::diffattn_launch<1, 2>(p, cache_f32, dim3(B, H, splits), stream);
+    if (rc == 0 && splits > 1) lgs::diffattn_combine_kernel<2><<<dim3(B, H), 256, 0, stream>>>(p, splits);
   } else {
     p.tiles = (max_len + 7) / 8;
     LGA_CHECK_ARG((long)B * p.tiles < (1L << 31), "lgs_diffattn: too many tiles");
-    rc = lgs::diffattn_launch<8>(p, cache_f32, dim3(B * p.tiles, H, 1), stream);
+    rc = lgs::diffattn_launch<8, 2>(p, cache_f32, dim3(B * p.tiles, H, 1), stream);
+  }
+  if (rc) return rc;
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_normattn_prepare(float* proj, long ld, int q_off, int k_off, int v_off, void* cache_k, void* cache_v,
+                                    int cache_f32, const int* slot, const int* pos, int T, int H, int G, int d, int dv,
+                                    int max_seq, float eps, float temp_coef, int temp_every, hipStream_t stream) {
+  LGA_CHECK_ARG(proj && slot && pos && cache_k && cache_v && T > 0 && max_seq > 0, "lgs_normattn_prepare: bad arguments");
+  LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && temp_every >= 0,
+                "lgs_normattn_prepare: heads must be a multiple of the key heads");
+  LGA_CHECK_ARG(q_off >= 0 && q_off + (long)H * d <= ld && k_off >= 0 && k_off + (long)G * d <= ld && v_off >= 0 &&
+                    v_off + (long)G * dv <= ld,
+                "lgs_normattn_prepare: queries, keys or values outside the row");
+  lgs::NormPrepArgs p{proj, ld, q_off, k_off, v_off, cache_k, cache_v, slot, pos, H, G, d, dv, max_seq, temp_every, eps, temp_coef};
+  if (cache_f32) lgs::normattn_prepare_kernel<true><<<T, 256, 0, stream>>>(p);
+  else lgs::normattn_prepare_kernel<false><<<T, 256, 0, stream>>>(p);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_sinkattn(const float* q, long ld, const void* cache_k, const void* cache_v, int cache_f32,
+                            const float* sink, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
+                            void* out_bf16, float* part, int splits, int B, int max_len, int H, int G, int d, int dv,
+                            int max_seq, int chunk, float scale, float cap, float post, hipStream_t stream) {
+  LGA_CHECK_ARG(q && cache_k && cache_v && seq_start && seq_slot && seq_pos0 && out, "lgs_sinkattn: null pointer");
+  LGA_CHECK_ARG(B > 0 && max_len > 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0, "lgs_sinkattn: bad sizes");
+  LGA_CHECK_ARG(d > 0 && d <= 512 && dv > 0 && dv <= 256, "lgs_sinkattn: key dim <= 512, value dim <= 256");
+  LGA_CHECK_ARG(ld >= (long)H * d && chunk >= 0 && max_seq > 0, "lgs_sinkattn: bad sizes");
+  LGA_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || (part && max_len == 1)),
+                "lgs_sinkattn: splits need one token per sequence and a workspace");
+  lgs::AttnArgs p{q, ld, cache_k, cache_v, seq_start, seq_slot, seq_pos0, out, (uint16_t*)out_bf16, part,
+                  H, G, d, dv, max_seq, chunk, 0, scale, cap, 0.0f, 0.0f, post, sink};
+  int rc;
+  if (max_len == 1) {
+    p.tiles = 1;
+    rc = lgs::diffattn_launch<1, 1>(p, cache_f32, dim3(B, H, splits), stream);
+    if (rc == 0 && splits > 1) lgs::diffattn_combine_kernel<1><<<dim3(B, H), 256, 0, stream>>>(p, splits);
+  } else {
+    p.tiles = (max_len + 15) / 16;
+    LGA_CHECK_ARG((long)B * p.tiles < (1L << 31), "lgs_sinkattn: too many tiles");
+    rc = lgs::diffattn_launch<16, 1>(p, cache_f32, dim3(B * p.tiles, H, 1), stream);
   }
   if (rc) return rc;
   LGA_LAUNCH_RETURN();

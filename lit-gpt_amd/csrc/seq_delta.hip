@@ -1,0 +1,250 @@
+// Gated delta rule of the layered models: a per-head outer-product memory S (d x dv, fp32, one per cache slot) that is
+// decayed, corrected towards the value of the current key, and read by the query:
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// g is one number per head, or one per head and key channel (the rows of S). Query / key heads may be shared by
+// groups of value heads (head h reads q / k head h / (H / G)). Everything that enters the recurrence is fp32.
+//
+//   lgs_delta_prepare   per token: q and k (after their convolution) become unit vectors per head, q times q_scale;
+//                       beta = sigmoid(raw); g = exp(-exp(A_log) softplus(raw + dt_bias))
+//   lgs_gated_delta     the recurrence, token by token for every step kind. The columns of S never mix, so a column
+//                       is owned by LPC adjacent lanes that hold d / LPC of its rows in registers; the two dot
+//                       products over the rows are summed inside those lanes with DPP adds (no LDS, no barrier);
+//                       q, k, g, v, beta of 16 tokens at a time are staged in LDS, the next 16 prefetched in registers
+//                       (8 at a time for key dims above 256)
+#include "seq_common.h"
+
+namespace lgs {
+
+__device__ __forceinline__ float softplus_d(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+struct DeltaPrepArgs {
+  float* qkv;  // [T][ld]: q [G][d] | k [G][d] | v [H][dv] after the convolution; q and k are normalised in place
+  long ld;
+  const float* a;  // raw decay inputs, row stride lda: [H][d] (per_channel) or [H]
+  long lda;
+  const float* b;  // raw beta inputs [H], row stride ldb
+  long ldb;
+  const float *A_log, *dt_bias;  // [H]; [H][d] or [H]
+  float* dec;                    // [T][H][d] or [T][H]
+  float* beta;                   // [T][H]
+  int H, G, d, per_channel;
+  float q_scale, norm_eps;
+};
+
+// grid (T): wave w makes the vectors w, w + 4, ... of the 2 G query / key heads unit vectors; all threads walk the
+// decays and betas
+__global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
+  const size_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int d = p.d;
+  float* row = p.qkv + t * p.ld;
+  for (int vec = wave; vec < 2 * p.G; vec += 4) {
+    float* x = row + (size_t)vec * d;
+    float ss = 0.0f;
+    for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
+    ss = wave_sum(ss);
+    const float s = (vec < p.G ? p.q_scale : 1.0f) / sqrtf(ss + p.norm_eps);
+    for (int i = lane; i < d; i += 64) x[i] *= s;
+  }
+  const int dc = p.per_channel ? d : 1, n = p.H * dc;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float rate = expf(p.A_log[i / dc]);
+    p.dec[t * n + i] = expf(-rate * softplus_d(p.a[t * p.lda + i] + p.dt_bias[i]));
+  }
+  for (int h = threadIdx.x; h < p.H; h += 256) p.beta[t * p.H + h] = sigmoid_f(p.b[t * p.ldb + h]);
+}
+
+struct DeltaArgs {
+  const float* qkv;  // [T][ld]: unit q [G][d] | unit k [G][d] | v [H][dv]
+  long ld;
+  const float* dec;   // [T][H][dc], dc = d or 1
+  const float* beta;  // [T][H]
+  float* state;       // [slots][H][d][dv]
+  const int *seq_start, *seq_slot, *seq_pos0;
+  float* out;  // [T][H * dv]
+  int H, G, d, dv, per_channel;
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// sum over LPC adjacent lanes (aligned, inside a row of 16 lanes); every lane of the group gets the sum. The order
+// of the additions is fixed: neighbours, pairs, then the mirrored halves.
+template <int LPC>
+__device__ __forceinline__ float lanes_sum(float v) {
+  v += dpp_f<0xB1>(v);                  // quad_perm [1, 0, 3, 2]
+  v += dpp_f<0x4E>(v);                  // quad_perm [2, 3, 0, 1]
+  if (LPC >= 8) v += dpp_f<0x141>(v);   // row_half_mirror: lane i of 8 with lane 7 - i
+  if (LPC >= 16) v += dpp_f<0x140>(v);  // row_mirror: lane i of 16 with lane 15 - i
+  return v;
+}
+
+
+// grid (ceil(dv / CW), H, B), CW = 256 / LPC columns per workgroup. Lane l of a wave: r = l % LPC, column
+// l / LPC of the wave's 64 / LPC; the lane holds the rows 4 (r + LPC j) + e, j < NR4, e < 4, of its column.
+template <int NR4, int LPC>
+__global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
+  constexpr int DP = 4 * NR4 * LPC;      // rows, padded
+  constexpr int CW = 256 / LPC;          // columns per workgroup
+  constexpr int ROW = 3 * DP + CW + 4;   // staged floats per token: q | k | g | v | beta (rows stay 16-byte aligned)
+  constexpr int kDeltaTB = DP > 256 ? 8 : 16;  // tokens staged at a time
+  constexpr int PRE = (kDeltaTB * ROW + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float st[kDeltaTB * ROW];
+  __shared__ float os[kDeltaTB][CW];
+  const int tid = threadIdx.x;
+  const int r = tid % LPC, cw = tid / LPC;  // cw: column inside the workgroup
+  const int hd = blockIdx.y, b = blockIdx.z;
+  const int col = blockIdx.x * CW + cw;
+  const int d = p.d, dv = p.dv, H = p.H;
+  const bool live = col < dv;
+  const int g = hd / (H / p.G);
+  const int r0 = p.seq_start[b], n = p.seq_start[b + 1] - r0;
+  const int dc = p.per_channel ? d : 1;
+  float* sp = p.state + (((size_t)p.seq_slot[b] * H + hd) * d) * dv;
+  const bool fresh = p.seq_pos0[b] == 0;
+  float S[NR4][4];
+#pragma unroll
+  for (int j = 0; j < NR4; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int row = 4 * (r + LPC * j) + e;
+      S[j][e] = (!fresh && live && row < d) ? sp[(size_t)row * dv + col] : 0.0f;
+    }
+  const size_t qo = (size_t)g * d, ko = (size_t)(p.G + g) * d, vo = (size_t)2 * p.G * d + (size_t)hd * dv + blockIdx.x * CW;
+
+  // staged item idx of the batch that starts at token t0: token idx / ROW, entry idx % ROW
+  auto fetch = [&](int t0, int idx) -> float {
+    const int t = idx / ROW, e = idx % ROW;
+    if (idx >= kDeltaTB * ROW || t0 + t >= n) return 0.0f;
+    const size_t rw = (size_t)(r0 + t0 + t);
+    if (e < DP) return e < d ? p.qkv[rw * p.ld + qo + e] : 0.0f;
+    if (e < 2 * DP) return e - DP < d ? p.qkv[rw * p.ld + ko + (e - DP)] : 0.0f;
+    if (e < 3 * DP) {
+      const int c = e - 2 * DP;
+      return c < d ? p.dec[(rw * H + hd) * dc + (dc == 1 ? 0 : c)] : 1.0f;
+    }
+    if (e < 3 * DP + CW) {
+      const int c = e - 3 * DP;
+      return blockIdx.x * CW + c < dv ? p.qkv[rw * p.ld + vo + c] : 0.0f;
+    }
+    return p.beta[rw * H + hd];
+  };
+  float pre[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) pre[i] = fetch(0, tid + 256 * i);
+
+  for (int t0 = 0; t0 < n; t0 += kDeltaTB) {
+    const int nb = min(kDeltaTB, n - t0);
+    __syncthreads();  // the previous batch's reads of st and os are done
+#pragma unroll
+    for (int i = 0; i < PRE; ++i)
+      if (tid + 256 * i < kDeltaTB * ROW) st[tid + 256 * i] = pre[i];
+    __syncthreads();
+    if (t0 + kDeltaTB < n) {
+#pragma unroll
+      for (int i = 0; i < PRE; ++i) pre[i] = fetch(t0 + kDeltaTB, tid + 256 * i);
+    }
+    for (int t = 0; t < nb; ++t) {
+      const float* row = st + t * ROW;
+      float ks = 0.0f;
+      float4 k4[NR4];
+#pragma unroll
+      for (int j = 0; j < NR4; ++j) {
+        const int at = 4 * (r + LPC * j);
+        k4[j] = *(const float4*)(row + DP + at);
+        const float4 g4 = *(const float4*)(row + 2 * DP + at);
+        S[j][0] *= g4.x;
+        S[j][1] *= g4.y;
+        S[j][2] *= g4.z;
+        S[j][3] *= g4.w;
+        ks = fmaf(S[j][0], k4[j].x, ks);
+        ks = fmaf(S[j][1], k4[j].y, ks);
+        ks = fmaf(S[j][2], k4[j].z, ks);
+        ks = fmaf(S[j][3], k4[j].w, ks);
+      }
+      ks = lanes_sum<LPC>(ks);
+      const float u = row[3 * DP + CW] * (row[3 * DP + cw] - ks);
+      float o = 0.0f;
+#pragma unroll
+      for (int j = 0; j < NR4; ++j) {
+        const float4 q4 = *(const float4*)(row + 4 * (r + LPC * j));
+        S[j][0] = fmaf(k4[j].x, u, S[j][0]);
+        S[j][1] = fmaf(k4[j].y, u, S[j][1]);
+        S[j][2] = fmaf(k4[j].z, u, S[j][2]);
+        S[j][3] = fmaf(k4[j].w, u, S[j][3]);
+        o = fmaf(S[j][0], q4.x, o);
+        o = fmaf(S[j][1], q4.y, o);
+        o = fmaf(S[j][2], q4.z, o);
+        o = fmaf(S[j][3], q4.w, o);
+      }
+      o = lanes_sum<LPC>(o);
+      if (r == 0) os[t][cw] = o;
+    }
+    __syncthreads();
+    for (int i = tid; i < nb * CW; i += 256) {
+      const int t = i / CW, c = i % CW;
+      if (blockIdx.x * CW + c < dv)
+        p.out[(size_t)(r0 + t0 + t) * H * dv + (size_t)hd * dv + blockIdx.x * CW + c] = os[t][c];
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < NR4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int row = 4 * (r + LPC * j) + e;
+        if (row < d) sp[(size_t)row * dv + col] = S[j][e];
+      }
+  }
+}
+
+template <int LPC>
+static bool gated_delta_launch(const DeltaArgs& p, int B, hipStream_t stream) {
+  const dim3 grid((p.dv + 256 / LPC - 1) / (256 / LPC), p.H, B);
+  const int nr4 = (p.d + 4 * LPC - 1) / (4 * LPC);
+  if (nr4 <= 1) gated_delta_kernel<1, LPC><<<grid, 256, 0, stream>>>(p);
+  else if (nr4 <= 2) gated_delta_kernel<2, LPC><<<grid, 256, 0, stream>>>(p);
+  else if (nr4 <= 4) gated_delta_kernel<4, LPC><<<grid, 256, 0, stream>>>(p);
+  else if (nr4 <= 8) gated_delta_kernel<8, LPC><<<grid, 256, 0, stream>>>(p);
+  else return false;
+  return true;
+}
+
+}  // namespace lgs
+
+extern "C" int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb,
+                                 const float* A_log, const float* dt_bias, float* dec, float* beta, int T, int H, int G,
+                                 int d, int per_channel, float q_scale, float norm_eps, hipStream_t stream) {
+  LGA_CHECK_ARG(qkv && a && b && A_log && dt_bias && dec && beta && T > 0, "lgs_delta_prepare: bad arguments");
+  LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && ld >= 2L * G * d, "lgs_delta_prepare: bad sizes");
+  lgs::DeltaPrepArgs p{qkv, ld, a, lda, b, ldb, A_log, dt_bias, dec, beta, H, G, d, per_channel ? 1 : 0, q_scale, norm_eps};
+  lgs::delta_prepare_kernel<<<T, 256, 0, stream>>>(p);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, float* state,
+                               const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, int B, int H,
+                               int G, int d, int dv, int per_channel, int lanes, hipStream_t stream) {
+  LGA_CHECK_ARG(qkv && dec && beta && state && seq_start && seq_slot && seq_pos0 && out, "lgs_gated_delta: null pointer");
+  LGA_CHECK_ARG(B > 0 && B <= 65535 && H > 0 && H <= 65535 && G > 0 && H % G == 0 && d > 0 && d <= 512 && dv > 0,
+                "lgs_gated_delta: bad sizes (key dim <= 512)");
+  LGA_CHECK_ARG(ld >= 2L * G * d + (long)H * dv, "lgs_gated_delta: q | k | v outside the row");
+  lgs::DeltaArgs p{qkv, ld, dec, beta, state, seq_start, seq_slot, seq_pos0, out, H, G, d, dv, per_channel ? 1 : 0};
+  // lanes per column: more lanes shorten a token's dependent chain and multiply the waves; by default as many as
+  // keep the launch within about two waves per SIMD, and at least enough for 32 rows per lane
+  int lpc = lanes;
+  if (lpc == 0) {
+    const long cols = (long)B * H * dv;
+    lpc = cols * 16 / 64 <= 2048 ? 16 : cols * 8 / 64 <= 2048 ? 8 : 4;
+    while (lpc > 4 && 4 * lpc > d) lpc >>= 1;
+  }
+  while (lpc < 16 && d > 32 * lpc) lpc <<= 1;
+  bool ok;
+  if (lpc == 4) ok = lgs::gated_delta_launch<4>(p, B, stream);
+  else if (lpc == 8) ok = lgs::gated_delta_launch<8>(p, B, stream);
+  else if (lpc == 16) ok = lgs::gated_delta_launch<16>(p, B, stream);
+  else ok = false;
+  LGA_CHECK_ARG(ok, "lgs_gated_delta: lanes per column must be 4, 8 or 16 and cover the key dim");
+  LGA_LAUNCH_RETURN();
+}

@@ -4,6 +4,8 @@
 //   lgs_glu_clamped      out = g sigmoid(alpha g) (u + shift) with g = min(a, limit), u = clamp(b, -limit, limit)
 //   lgs_moe_route        per token: the `top` largest router logits (fp32, lowest index first among equals) and the
 //                        softmax over just those
+//   lgs_moe_route_scores per token: softmax over all router outputs; the choice adds a stored correction to the
+//                        scores, the weights are the chosen scores themselves
 //   lgs_moe_up / _down   the routed experts as streaming GEMVs over (token, choice) pairs: only the chosen experts'
 //                        rows are read; the down kernel sums a token's choices in their routing order and adds the
 //                        result to the residual stream (the decode form; a prompt runs grouped products instead)
@@ -16,8 +18,8 @@ namespace lgs {
 
 __global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ a, const float* __restrict__ b, long ld,
                                                   float* __restrict__ out, uint16_t* __restrict__ out16, int n, int act) {
-  const size_t t = blockIdx.y;
-  const int i = blockIdx.x * 256 + threadIdx.x;
+  const size_t t = blockIdx.x;
+  const int i = blockIdx.y * 256 + threadIdx.x;
   if (i >= n) return;
   const float v = act_f(act, a[t * ld + i]) * b[t * ld + i];
   if (out16) out16[t * n + i] = f2bf(v);  // the operand of a bf16 product: rounded here instead of at its load
@@ -86,17 +88,79 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__
     for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= den;
 }
 
-// grid (ceil(F / 8), pairs): pair = token * top + choice; act[pair][f] = act(up_e[f] . h_token)
-template <bool WF32>
+// one wave per token: s = softmax(z) over all E outputs; the `top` largest of s + bias (lowest index first among
+// equals) are chosen, and their weights are s itself: not renormalised, without the bias
+__global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* __restrict__ z, long ld, int E, int top,
+                                                              const float* __restrict__ bias, int* __restrict__ ids,
+                                                              float* __restrict__ wts) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  float s[4], c[4], mx = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    s[e] = lane + 64 * e < E ? z[(size_t)t * ld + lane + 64 * e] : -INFINITY;
+    mx = fmaxf(mx, s[e]);
+  }
+  mx = wave_max(mx);
+  float den = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    s[e] = lane + 64 * e < E ? expf(s[e] - mx) : 0.0f;
+    den += s[e];
+  }
+  den = wave_sum(den);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int i = lane + 64 * e;
+    s[e] /= den;
+    c[e] = i < E ? s[e] + (bias ? bias[i] : 0.0f) : -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY, bs = 0.0f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = lane + 64 * e;
+      if (i < E && (c[e] > best || (c[e] == best && i < bi))) {
+        best = c[e];
+        bs = s[e];
+        bi = i;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o), os = __shfl_xor(bs, o);
+      const int oi = __shfl_xor(bi, o);
+      if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bs = os;
+        bi = oi;
+      }
+    }
+    if (lane == 0) {
+      ids[(size_t)t * top + k] = bi;
+      wts[(size_t)t * top + k] = bs;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (lane + 64 * e == bi) c[e] = -INFINITY;
+  }
+}
+
+// grid (ceil(F / 8), pairs): pair = token * top + choice; act[pair][f] = act(up_e[f] . h_token); GATED: an expert's
+// matrix holds F gate rows, then F up rows, and act[pair][f] = act(gate_e[f] . h) * (up_e[f] . h), 4 per workgroup.
+// Pairs whose expert id is >= n_real (experts without matrices) are skipped.
+template <bool WF32, bool GATED>
 __global__ void __launch_bounds__(256) moe_up_kernel(const float* __restrict__ h, long ldh, const void* __restrict__ up,
                                                      const int* __restrict__ ids, float* __restrict__ actbuf, int top,
-                                                     int F, int K, int act) {
+                                                     int F, int K, int act, int n_real) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pair = blockIdx.y, f0 = (blockIdx.x * 4 + wave) * 2;
+  const int pair = blockIdx.y, f0 = (blockIdx.x * 4 + wave) * (GATED ? 1 : 2);
   if (f0 >= F) return;
   const int e = ids[pair];
+  if (e >= n_real) return;
   const float* hr = h + (size_t)(pair / top) * ldh;
-  const size_t w0 = ((size_t)e * F + f0) * K, w1 = ((size_t)e * F + min(f0 + 1, F - 1)) * K;
+  const size_t rows = GATED ? 2 * (size_t)F : (size_t)F;
+  const size_t w0 = ((size_t)e * rows + f0) * K, w1 = ((size_t)e * rows + (GATED ? F + f0 : min(f0 + 1, F - 1))) * K;
   float a0 = 0.0f, a1 = 0.0f;
   for (int k = lane; k < K; k += 64) {
     const float x = aop<WF32>(hr[k]);
@@ -106,22 +170,35 @@ __global__ void __launch_bounds__(256) moe_up_kernel(const float* __restrict__ h
   a0 = wave_sum(a0);
   a1 = wave_sum(a1);
   if (lane == 0) {
-    actbuf[(size_t)pair * F + f0] = act_f(act, a0);
-    if (f0 + 1 < F) actbuf[(size_t)pair * F + f0 + 1] = act_f(act, a1);
+    if (GATED) {
+      actbuf[(size_t)pair * F + f0] = act_f(act, a0) * a1;
+    } else {
+      actbuf[(size_t)pair * F + f0] = act_f(act, a0);
+      if (f0 + 1 < F) actbuf[(size_t)pair * F + f0 + 1] = act_f(act, a1);
+    }
   }
 }
 
-// grid (ceil(N / 8), T): x[t][n] += sum_k wts[t][k] * (down_e(t,k)[n] . act[t * top + k]), k ascending
+// grid (ceil(N / 8), T): x[t][n] (+)= sum_k wts[t][k] * (down_e(t,k)[n] . act[t * top + k]), k ascending; an expert
+// id >= n_real is an identity expert: its output is the token's input hin[t][n] itself
 template <bool WF32>
 __global__ void __launch_bounds__(256) moe_down_kernel(const float* __restrict__ actbuf, const void* __restrict__ down,
                                                        const int* __restrict__ ids, const float* __restrict__ wts,
-                                                       float* __restrict__ x, long ldx, int top, int N, int F) {
+                                                       float* __restrict__ x, long ldx, int top, int N, int F,
+                                                       int n_real, const float* __restrict__ hin, long ldh,
+                                                       int accumulate) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.y, n0 = (blockIdx.x * 4 + wave) * 2;
   if (n0 >= N) return;
   float y0 = 0.0f, y1 = 0.0f;
   for (int k = 0; k < top; ++k) {
     const int e = ids[(size_t)t * top + k];
+    if (e >= n_real) {  // (the whole wave takes this branch)
+      const float w = wts[(size_t)t * top + k];
+      y0 = fmaf(w, hin[(size_t)t * ldh + n0], y0);
+      y1 = fmaf(w, hin[(size_t)t * ldh + min(n0 + 1, N - 1)], y1);
+      continue;
+    }
     const float* ar = actbuf + ((size_t)t * top + k) * F;
     const size_t w0 = ((size_t)e * N + n0) * F, w1 = ((size_t)e * N + min(n0 + 1, N - 1)) * F;
     float a0 = 0.0f, a1 = 0.0f;
@@ -135,8 +212,8 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const float* __restrict__
     y1 = fmaf(w, wave_sum(a1), y1);
   }
   if (lane == 0) {
-    x[(size_t)t * ldx + n0] += y0;
-    if (n0 + 1 < N) x[(size_t)t * ldx + n0 + 1] += y1;
+    x[(size_t)t * ldx + n0] = accumulate ? x[(size_t)t * ldx + n0] + y0 : y0;
+    if (n0 + 1 < N) x[(size_t)t * ldx + n0 + 1] = accumulate ? x[(size_t)t * ldx + n0 + 1] + y1 : y1;
   }
 }
 
@@ -195,15 +272,21 @@ __global__ void __launch_bounds__(256) moe_place_kernel(const int* __restrict__ 
   }
 }
 
-// grid (ceil(N / 256), T): x[t] += sum_k wts[t][k] * y[where[t * top + k]], k ascending
+// grid (ceil(N / 256), T): x[t] (+)= sum_k wts[t][k] * y[where[t * top + k]], k ascending; with ids, a choice whose
+// expert id is >= n_real (an identity expert) contributes the token's input hin[t] instead of a row of y
 __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ where,
                                                           const float* __restrict__ wts, float* __restrict__ x, long ldx,
-                                                          int top, int N) {
+                                                          int top, int N, const int* __restrict__ ids, int n_real,
+                                                          const float* __restrict__ hin, long ldh, int accumulate) {
   const int t = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
   if (n >= N) return;
   float s = 0.0f;
-  for (int k = 0; k < top; ++k) s = fmaf(wts[(size_t)t * top + k], y[(size_t)where[(size_t)t * top + k] * N + n], s);
-  x[(size_t)t * ldx + n] += s;
+  for (int k = 0; k < top; ++k) {
+    const size_t pair = (size_t)t * top + k;
+    const float v = ids && ids[pair] >= n_real ? hin[(size_t)t * ldh + n] : y[(size_t)where[pair] * N + n];
+    s = fmaf(wts[pair], v, s);
+  }
+  x[(size_t)t * ldx + n] = accumulate ? x[(size_t)t * ldx + n] + s : s;
 }
 
 // grid (T): LDS holds the row x (W floats), the gated slice (dim floats) and the projection y (W floats)
@@ -247,8 +330,8 @@ __global__ void __launch_bounds__(256) token_side_kernel(float* __restrict__ x, 
 
 extern "C" int lgs_glu(const float* a, const float* b, long ld, void* out, int out_bf16, int T, int n, int act,
                        hipStream_t stream) {
-  LGA_CHECK_ARG(a && b && out && T > 0 && T <= 65535 && n > 0, "lgs_glu: bad arguments");
-  lgs::glu_kernel<<<dim3((n + 255) / 256, T), 256, 0, stream>>>(a, b, ld, out_bf16 ? nullptr : (float*)out,
+  LGA_CHECK_ARG(a && b && out && T > 0 && n > 0 && (n + 255) / 256 <= 65535, "lgs_glu: bad arguments");
+  lgs::glu_kernel<<<dim3(T, (n + 255) / 256), 256, 0, stream>>>(a, b, ld, out_bf16 ? nullptr : (float*)out,
                                                                  out_bf16 ? (uint16_t*)out : nullptr, n, act);
   LGA_LAUNCH_RETURN();
 }
@@ -269,23 +352,43 @@ extern "C" int lgs_moe_route(const float* z, long ld, int T, int E, int top, int
   LGA_LAUNCH_RETURN();
 }
 
+extern "C" int lgs_moe_route_scores(const float* z, long ld, int T, int E, int top, const float* bias, int* ids,
+                                    float* wts, hipStream_t stream) {
+  LGA_CHECK_ARG(z && ids && wts && T > 0, "lgs_moe_route_scores: bad arguments");
+  LGA_CHECK_ARG(E > 0 && E <= 256 && top > 0 && top <= E,
+                "lgs_moe_route_scores: experts must be <= 256 and top <= experts");
+  lgs::moe_route_scores_kernel<<<T, 64, 0, stream>>>(z, ld, E, top, bias, ids, wts);
+  LGA_LAUNCH_RETURN();
+}
+
 extern "C" int lgs_moe_up(const float* h, long ldh, const void* up, int w_f32, const int* ids, float* actbuf, int T,
-                          int top, int F, int K, int act, hipStream_t stream) {
-  LGA_CHECK_ARG(h && up && ids && actbuf && T > 0 && top > 0 && F > 0 && K > 0 && (long)T * top <= 65535,
+                          int top, int F, int K, int act, int gated, int n_real, hipStream_t stream) {
+  LGA_CHECK_ARG(h && up && ids && actbuf && T > 0 && top > 0 && F > 0 && K > 0 && (long)T * top <= 65535 && n_real > 0,
                 "lgs_moe_up: bad arguments");
-  const dim3 grid((F + 7) / 8, T * top);
-  if (w_f32) lgs::moe_up_kernel<true><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act);
-  else lgs::moe_up_kernel<false><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act);
+  if (gated) {
+    const dim3 grid((F + 3) / 4, T * top);
+    if (w_f32) lgs::moe_up_kernel<true, true><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act, n_real);
+    else lgs::moe_up_kernel<false, true><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act, n_real);
+  } else {
+    const dim3 grid((F + 7) / 8, T * top);
+    if (w_f32) lgs::moe_up_kernel<true, false><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act, n_real);
+    else lgs::moe_up_kernel<false, false><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act, n_real);
+  }
   LGA_LAUNCH_RETURN();
 }
 
 extern "C" int lgs_moe_down(const float* actbuf, const void* down, int w_f32, const int* ids, const float* wts,
-                            float* x, long ldx, int T, int top, int N, int F, hipStream_t stream) {
-  LGA_CHECK_ARG(actbuf && down && ids && wts && x && T > 0 && T <= 65535 && top > 0 && N > 0 && F > 0,
+                            float* x, long ldx, int T, int top, int N, int F, int n_real, const float* hin, long ldh,
+                            int accumulate, hipStream_t stream) {
+  LGA_CHECK_ARG(actbuf && down && ids && wts && x && T > 0 && T <= 65535 && top > 0 && N > 0 && F > 0 && n_real > 0 && hin,
                 "lgs_moe_down: bad arguments");
   const dim3 grid((N + 7) / 8, T);
-  if (w_f32) lgs::moe_down_kernel<true><<<grid, 256, 0, stream>>>(actbuf, down, ids, wts, x, ldx, top, N, F);
-  else lgs::moe_down_kernel<false><<<grid, 256, 0, stream>>>(actbuf, down, ids, wts, x, ldx, top, N, F);
+  if (w_f32)
+    lgs::moe_down_kernel<true><<<grid, 256, 0, stream>>>(actbuf, down, ids, wts, x, ldx, top, N, F, n_real, hin, ldh,
+                                                         accumulate);
+  else
+    lgs::moe_down_kernel<false><<<grid, 256, 0, stream>>>(actbuf, down, ids, wts, x, ldx, top, N, F, n_real, hin, ldh,
+                                                          accumulate);
   LGA_LAUNCH_RETURN();
 }
 
@@ -301,9 +404,12 @@ extern "C" int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_st
 }
 
 extern "C" int lgs_moe_combine(const float* y, const int* where, const float* wts, float* x, long ldx, int T, int top,
-                               int N, hipStream_t stream) {
+                               int N, const int* ids, int n_real, const float* hin, long ldh, int accumulate,
+                               hipStream_t stream) {
   LGA_CHECK_ARG(y && where && wts && x && T > 0 && T <= 65535 && top > 0 && N > 0, "lgs_moe_combine: bad arguments");
-  lgs::moe_combine_kernel<<<dim3((N + 255) / 256, T), 256, 0, stream>>>(y, where, wts, x, ldx, top, N);
+  LGA_CHECK_ARG(!ids || hin, "lgs_moe_combine: identity experts need the tokens' inputs");
+  lgs::moe_combine_kernel<<<dim3((N + 255) / 256, T), 256, 0, stream>>>(y, where, wts, x, ldx, top, N, ids, n_real, hin,
+                                                                          ldh, accumulate);
   LGA_LAUNCH_RETURN();
 }
 

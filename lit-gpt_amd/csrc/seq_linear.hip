@@ -319,6 +319,72 @@ __global__ void __launch_bounds__(256) embed_kernel(const int* __restrict__ tok,
   for (int i = threadIdx.x; i < W; i += 256) x[(size_t)t * W + i] = wload<WF32>(table, (size_t)id * W + i) * scale;
 }
 
+// x[t] = table[tok[t]] * scale + ptable[pos[t]] (a learned position vector, not scaled); x16: optional rounded copy
+template <bool WF32>
+__global__ void __launch_bounds__(256) embed_pos_kernel(const int* __restrict__ tok, const int* __restrict__ pos,
+                                                        const void* __restrict__ table, const void* __restrict__ ptable,
+                                                        float* __restrict__ x, uint16_t* __restrict__ x16, int W, int vocab,
+                                                        int positions, float scale) {
+  const int t = blockIdx.x;
+  int id = tok[t], ps = pos[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host validates ids and positions
+  ps = ps < 0 ? 0 : (ps >= positions ? positions - 1 : ps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = fmaf(wload<WF32>(table, (size_t)id * W + i), scale, wload<WF32>(ptable, (size_t)ps * W + i));
+    x[(size_t)t * W + i] = v;
+    if (x16) x16[(size_t)t * W + i] = f2bf(v);
+  }
+}
+
+// Layer norm of a sublayer's output joining the residual: x[r] (+)= mult * ((y - mean) / sqrt(var + eps) * w + b),
+// var = mean of the squared deviations (two passes over the row, which stays in registers up to 256 * CPT columns).
+// x16: optional copy of the new x rounded to bf16 (the next product's operand). grid (rows).
+template <int CPT>
+__global__ void __launch_bounds__(256) layernorm_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                        const float* __restrict__ b, float eps, float mult, int accumulate,
+                                                        float* __restrict__ x, uint16_t* __restrict__ x16, int n) {
+  __shared__ float red[4];
+  const size_t r = blockIdx.x;
+  const float* yr = y + r * n;
+  float v[CPT];
+  float s = 0.0f;
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) {
+    const int i = threadIdx.x + 256 * e;
+    v[e] = i < n ? yr[i] : 0.0f;
+    s += v[e];
+  }
+  for (int i = threadIdx.x + 256 * CPT; i < n; i += 256) s += yr[i];
+  const float mean = block_sum_256(s, red) / (float)n;
+  float q = 0.0f;
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) {
+    const float dlt = threadIdx.x + 256 * e < n ? v[e] - mean : 0.0f;
+    q = fmaf(dlt, dlt, q);
+  }
+  for (int i = threadIdx.x + 256 * CPT; i < n; i += 256) {
+    const float dlt = yr[i] - mean;
+    q = fmaf(dlt, dlt, q);
+  }
+  const float rstd = 1.0f / sqrtf(block_sum_256(q, red) / (float)n + eps);
+  auto put = [&](int i, float val) {
+    float o = mult * fmaf((val - mean) * rstd, w[i], b ? b[i] : 0.0f);
+    if (accumulate) o += x[r * n + i];
+    x[r * n + i] = o;
+    if (x16) x16[r * n + i] = f2bf(o);
+  };
+#pragma unroll
+  for (int e = 0; e < CPT; ++e)
+    if (threadIdx.x + 256 * e < n) put(threadIdx.x + 256 * e, v[e]);
+  for (int i = threadIdx.x + 256 * CPT; i < n; i += 256) put(i, yr[i]);
+}
+
+// z <- cap * tanh(z / cap)
+__global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, size_t n, float cap) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) z[i] = cap * tanhf(z[i] / cap);
+}
+
 // grid (rows, groups): group g of row r is x[r * ldx + g * n .. + n); weight (may be null) is indexed within a group
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, long ldx, const float* __restrict__ w,
                                                       float offset, float eps, float* __restrict__ y, long ldy, int n,
@@ -410,6 +476,36 @@ extern "C" int lgs_embed(const int* tokens, const void* table, int w_f32, float 
   LGA_CHECK_ARG(tokens && table && x && T > 0 && W > 0 && vocab > 0, "lgs_embed: bad arguments");
   if (w_f32) lgs::embed_kernel<true><<<T, 256, 0, stream>>>(tokens, table, x, W, vocab, scale);
   else lgs::embed_kernel<false><<<T, 256, 0, stream>>>(tokens, table, x, W, vocab, scale);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_embed_pos(const int* tokens, const int* pos, const void* table, const void* pos_table, int w_f32,
+                             float scale, float* x, void* x_bf16, int T, int W, int vocab, int positions,
+                             hipStream_t stream) {
+  LGA_CHECK_ARG(tokens && pos && table && pos_table && x && T > 0 && W > 0 && vocab > 0 && positions > 0,
+                "lgs_embed_pos: bad arguments");
+  if (w_f32)
+    lgs::embed_pos_kernel<true><<<T, 256, 0, stream>>>(tokens, pos, table, pos_table, x, (uint16_t*)x_bf16, W, vocab,
+                                                       positions, scale);
+  else
+    lgs::embed_pos_kernel<false><<<T, 256, 0, stream>>>(tokens, pos, table, pos_table, x, (uint16_t*)x_bf16, W, vocab,
+                                                        positions, scale);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_layernorm(const float* y, const float* weight, const float* bias, float eps, float mult,
+                             int accumulate, float* x, void* x_bf16, int rows, int n, hipStream_t stream) {
+  LGA_CHECK_ARG(y && weight && x && rows > 0 && n > 0, "lgs_layernorm: bad arguments");
+  if (n <= 1024)
+    lgs::layernorm_kernel<4><<<rows, 256, 0, stream>>>(y, weight, bias, eps, mult, accumulate, x, (uint16_t*)x_bf16, n);
+  else
+    lgs::layernorm_kernel<16><<<rows, 256, 0, stream>>>(y, weight, bias, eps, mult, accumulate, x, (uint16_t*)x_bf16, n);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_softcap(float* z, long n, float cap, hipStream_t stream) {
+  LGA_CHECK_ARG(z && n > 0 && cap > 0.0f, "lgs_softcap: bad arguments");
+  lgs::softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(z, (size_t)n, cap);
   LGA_LAUNCH_RETURN();
 }
 

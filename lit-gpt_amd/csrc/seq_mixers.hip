@@ -299,10 +299,12 @@ static size_t retention_chunk_lds(int d) {
   return (size_t)(2 * kRC * DP + kRC * kVS + kRC * kAS + DPAD * kVS + 66) * sizeof(float);
 }
 
-// grid (T, H): o[t][h][:] <- (unit ? o / rms(o) : o) * act(g[t * ldg + h * dv + :])
-// (o16: optional rounded copy, the operand of the out-projection's bf16 MFMA tiles)
+// grid (T, H): o[t][h][:] <- (unit ? o / rms(o) : o) * w[:] * act(g[t * ldg + h * dv + :]) * post
+// (w: optional weight shared by the heads; o16: optional rounded copy, the operand of the out-projection's bf16
+// MFMA tiles)
 __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, const float* __restrict__ g, long ldg,
                                                         int H, int dv, int unit, float eps, int act,
+                                                        const float* __restrict__ w, float post,
                                                         uint16_t* __restrict__ o16) {
   __shared__ float red[4];
   const int t = blockIdx.x, h = blockIdx.y;
@@ -316,7 +318,10 @@ __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, c
     rstd = 1.0f / sqrtf(ss / (float)dv + eps);
   }
   for (int i = threadIdx.x; i < dv; i += 256) {
-    const float v = orow[i] * rstd * act_f(act, grow[i]);
+    float v = orow[i] * rstd;
+    if (w) v *= w[i];
+    v *= act_f(act, grow[i]);
+    if (post != 1.0f) v *= post;
     orow[i] = v;
     if (o16) o16[((size_t)t * H + h) * dv + i] = f2bf(v);
   }
@@ -852,9 +857,10 @@ extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float*
 }
 
 extern "C" int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps,
-                             int act, void* o_bf16, hipStream_t stream) {
+                             int act, const float* weight, float post, void* o_bf16, hipStream_t stream) {
   LGA_CHECK_ARG(o && g && T > 0 && H > 0 && H <= 65535 && dv > 0, "lgs_head_gate: bad arguments");
-  lgs::head_gate_kernel<<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act, (uint16_t*)o_bf16);
+  lgs::head_gate_kernel<<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act, weight, post,
+                                                        (uint16_t*)o_bf16);
   LGA_LAUNCH_RETURN();
 }
 

@@ -178,7 +178,7 @@ class RotarySpec:
 
 @dataclass
 class MixerSpec:
-    kind: str  # "retention" | "latent_attention" | "attention" | "mamba2"
+    kind: str  # one of MIXER_KINDS
     heads: int
     dim: int  # per-head query / key size (latent attention: the unrotated part; attention: of one map)
     vdim: int
@@ -196,6 +196,14 @@ class MixerSpec:
     groups: int = 0  # mamba2: groups of heads that share B and C
     norm_groups: int = 1  # mamba2: equal parts of the gated output, each divided by its own root mean square
     state: int = 0  # mamba2: state size N
+    q_temp_coef: float = 0.0  # sink attention: the query is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)
+    q_temp_every: int = 0  # (0: no query temperature)
+    decay_rank: int = 0  # channel_delta: inner sizes of the low-rank decay and gate maps (a checkpoint's tensors give
+    gate_rank: int = 0  # them; these only size random weights, 0: 16)
+    left: Optional["MixerSpec"] = None  # parallel: two mixers that read the same input ...
+    right: Optional["MixerSpec"] = None
+    left_scale: float = 1.0  # ... and are summed with these factors
+    right_scale: float = 1.0
 
 
 @dataclass
@@ -205,6 +213,7 @@ class FeedForwardSpec:
     experts: int = 0
     top: int = 0
     limit: float = 0.0  # clamped gated unit: bound of the gate (from above) and of the up branch (both sides)
+    identity: int = 0  # moe: router outputs beyond ``experts`` that stand for identity experts (output = input)
 
 
 @dataclass
@@ -213,22 +222,35 @@ class LayerSpec:
     mlp: Optional[FeedForwardSpec]
 
 
-MIXER_KINDS = ("retention", "latent_attention", "attention", "mamba2")
+# "channel_delta" / "gated_delta": the gated delta rule with a decay per head and key channel / per head;
+# "sink_attention": softmax attention with unit-RMS queries and keys, a query temperature and a sink;
+# "parallel": a sink attention and a gated delta rule side by side
+MIXER_KINDS = ("retention", "latent_attention", "attention", "mamba2", "channel_delta", "gated_delta",
+               "sink_attention", "parallel")
 
 
 @dataclass(frozen=True)
 class LayeredDesign:
     """What a design fixes for all its models (everything else is in ``config.json``)."""
 
-    block: str  # "parallel": x += mixer(h) + ff(h), one norm; "sequential": x += mixer(norm1 x), then x += ff(norm2 x)
+    # "parallel": x += mixer(h) + ff(h), one norm; "sequential": x += mixer(norm1 x), then x += ff(norm2 x);
+    # "post": the sublayers read x itself and their OUTPUT is normed: x += m norm1(mixer(x)), then x += m norm2(ff(x))
+    block: str
     norm_offset: float  # the norm multiplies by offset + stored weight
     tied_head: bool  # logits from the embedding table itself, or from a matrix of their own ("head")
     dense_ff: str  # "gelu_tanh": W_down(gelu_tanh(gate) * up); "clamped_swish": g sigmoid(1.702 g) (u + 1), clamped
+    norm: str = "rms"  # "rms": x / rms(x) * w; "layer": (x - mean) / sqrt(var + eps) * w + b (tensor "<norm>.b")
+    positions: str = "none"  # "learned": a table "pos" whose row p joins the embedding at position p
+    # "top_logits": the largest router logits, softmax over the chosen, experts W_down relu(W_up h)^2;
+    # "scores": softmax over all router outputs (+ a stored correction for the choice only), weights = the chosen
+    # scores as they are, gated experts W_down(silu(W_gate h) * W_up h), optional identity experts
+    moe: str = "top_logits"
 
 
 DESIGNS: Dict[str, LayeredDesign] = {
     "Bavesun": LayeredDesign("parallel", 1.0, True, "gelu_tanh"),
     "Rigulorn": LayeredDesign("sequential", 0.0, False, "clamped_swish"),
+    "Ravelorn": LayeredDesign("post", 0.0, False, "gelu_tanh", norm="layer", positions="learned", moe="scores"),
 }
 
 
@@ -247,6 +269,9 @@ class LayeredConfig:
     name: str = ""
     streams: int = 1  # parallel residual streams (hyper-connections); 1 with no stream weights: the plain residual sum
     stream_weights: bool = False  # the checkpoint holds read / write / mix weights per sublayer
+    residual_mult: float = 1.0  # post-norm layers: factor of every normed sublayer output in the residual sum
+    logit_softcap: float = 0.0  # logits pass cap * tanh(z / cap) (0: not)
+    max_positions: int = 0  # rows of the learned position table (0: the design has none)
 
     @property
     def design(self) -> LayeredDesign:
@@ -261,10 +286,33 @@ class LayeredConfig:
         n = len(self.layers)
         if not (0 <= self.loop_start <= self.loop_stop <= n) or self.loop_times < 1:
             raise ValueError(f"loop [{self.loop_start}, {self.loop_stop}) x {self.loop_times} does not fit {n} layers")
+        if self.design.positions == "learned" and self.max_positions < 1:
+            raise ValueError("max_positions: the design adds a learned position vector")
         for i, spec in enumerate(self.layers):
             m = spec.mixer
             if m.kind not in MIXER_KINDS:
                 raise ValueError(f"layer {i}: unknown mixer {m.kind!r}")
+            if spec.mlp is not None and spec.mlp.kind == "moe":
+                f = spec.mlp
+                if not 0 < f.top <= f.experts + f.identity or f.identity < 0 or f.experts + f.identity > 256:
+                    raise ValueError(f"layer {i}: top {f.top} of {f.experts} + {f.identity} experts (at most 256)")
+            parts = [m.left, m.right] if m.kind == "parallel" else [m]
+            if m.kind == "parallel" and (m.left is None or m.left.kind != "sink_attention" or m.right is None or
+                                         m.right.kind != "gated_delta"):
+                raise ValueError(f"layer {i}: a parallel mixer holds a sink attention (left) and a gated delta rule (right)")
+            for q in parts:
+                if q.kind in ("channel_delta", "gated_delta"):
+                    if q.kv_heads < 1 or q.heads % q.kv_heads or not 1 <= q.dim <= 512 or q.vdim < 1:
+                        raise ValueError(f"layer {i}: heads {q.heads} / key heads {q.kv_heads} / key dim {q.dim} (<= 512)")
+                    if not 1 <= q.conv <= 16:
+                        raise ValueError(f"layer {i}: convolution taps 1..16 are served")
+                if q.kind == "sink_attention":
+                    if q.kv_heads < 1 or q.heads % q.kv_heads or not 1 <= q.dim <= 512 or not 1 <= q.vdim <= 256:
+                        raise ValueError(f"layer {i}: heads {q.heads} / key heads {q.kv_heads} / dims {q.dim}, {q.vdim}")
+                    if q.q_temp_every < 0:
+                        raise ValueError(f"layer {i}: q_temp.every must be positive")
+            if m.kind in ("channel_delta", "gated_delta", "sink_attention", "parallel"):
+                continue
             if m.kind == "retention" and (m.decay is None or len(m.decay) != m.heads):
                 raise ValueError(f"layer {i}: retention needs one decay per head")
             if m.kind == "mamba2":
@@ -285,8 +333,6 @@ class LayeredConfig:
                         raise ValueError(f"layer {i}: kv_from {j} must name an earlier attention layer with keys of its own")
                     if (src.kv_heads, src.dim, src.vdim) != (m.kv_heads, m.dim, m.vdim):
                         raise ValueError(f"layer {i}: its key heads and sizes differ from layer {j}'s")
-            if spec.mlp is not None and spec.mlp.kind == "moe" and not 0 < spec.mlp.top <= spec.mlp.experts:
-                raise ValueError(f"layer {i}: top {spec.mlp.top} of {spec.mlp.experts} experts")
 
     @property
     def layer_runs(self) -> List[int]:
@@ -295,30 +341,43 @@ class LayeredConfig:
         a, b = self.loop_start, self.loop_stop
         return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, len(self.layers)))
 
+    @staticmethod
+    def _mixer_spec(kind: str, m: Dict[str, Any]) -> MixerSpec:
+        if kind == "parallel":
+            return MixerSpec(kind=kind, heads=0, dim=0, vdim=0, rot=RotarySpec(),
+                             left=LayeredConfig._mixer_spec("sink_attention", m["left"]),
+                             right=LayeredConfig._mixer_spec("gated_delta", m["right"]),
+                             left_scale=float(m.get("left_scale", 1.0)), right_scale=float(m.get("right_scale", 1.0)))
+        rot = m.get("rot") or {}
+        mask = m.get("mask") or {}
+        temp = m.get("q_temp") or {}
+        return MixerSpec(kind=kind, heads=int(m["heads"]), dim=int(m.get("dim", 0)), vdim=int(m["vdim"]),
+                         rot=RotarySpec(int(rot.get("dims", 0)), float(rot.get("base", 10000.0))),
+                         decay=[float(x) for x in m["decay"]] if "decay" in m else None,
+                         kv_rank=int(m.get("kv_rank", 0)), rot_dim=int(m.get("rot_dim", 0)),
+                         scale=float(m.get("scale", 1.0)), kv_heads=int(m.get("kv_heads", m["heads"])),
+                         diff=float(m.get("diff", 0.0)), softcap=float(m.get("softcap") or 0.0),
+                         mask_size=int(mask.get("size") or 0),
+                         kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else None,
+                         conv=int(m.get("conv", 0)), groups=int(m.get("groups", 1)),
+                         norm_groups=int(m.get("norm_groups", 1)), state=int(m.get("state", 0)),
+                         q_temp_coef=float(temp.get("coef", 0.0)), q_temp_every=int(temp.get("every", 0)),
+                         decay_rank=int(m.get("decay_rank", 0)), gate_rank=int(m.get("gate_rank", 0)))
+
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "LayeredConfig":
         layers = []
         for entry in d["layers"]:
             m = entry["mixer"]
-            rot = m.get("rot") or {}
-            mask = m.get("mask") or {}
-            mixer = MixerSpec(kind=entry["type"], heads=int(m["heads"]), dim=int(m.get("dim", 0)), vdim=int(m["vdim"]),
-                              rot=RotarySpec(int(rot.get("dims", 0)), float(rot.get("base", 10000.0))),
-                              decay=[float(x) for x in m["decay"]] if "decay" in m else None,
-                              kv_rank=int(m.get("kv_rank", 0)), rot_dim=int(m.get("rot_dim", 0)),
-                              scale=float(m.get("scale", 1.0)), kv_heads=int(m.get("kv_heads", m["heads"])),
-                              diff=float(m.get("diff", 0.0)), softcap=float(m.get("softcap") or 0.0),
-                              mask_size=int(mask.get("size") or 0),
-                              kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else None,
-                              conv=int(m.get("conv", 0)), groups=int(m.get("groups", 1)),
-                              norm_groups=int(m.get("norm_groups", 1)), state=int(m.get("state", 0)))
+            mixer = cls._mixer_spec(entry["type"], m)
             f = entry.get("mlp")
             if f is None:
                 mlp = None
             elif f["kind"] == "dense":
                 mlp = FeedForwardSpec("dense", int(f["ff"]), limit=float(f.get("limit") or 0.0))
             elif f["kind"] == "moe":
-                mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]))
+                mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]),
+                                      identity=int(f["router"].get("identity") or 0))
             else:
                 raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
             layers.append(LayerSpec(mixer, mlp))
@@ -328,7 +387,9 @@ class LayeredConfig:
                    norm_eps=float(d["norm"]["eps"]), embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
                    layers=layers, loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
                    loop_times=int(loop.get("times", 1)), side_dim=int(side.get("dim", 0)),
-                   streams=int(d.get("streams", 1)), stream_weights="streams" in d)
+                   streams=int(d.get("streams", 1)), stream_weights="streams" in d,
+                   residual_mult=float(d.get("residual_mult", 1.0)), logit_softcap=float(d.get("logit_softcap") or 0.0),
+                   max_positions=int(d.get("max_positions") or 0))
 
     @classmethod
     def from_json(cls, path: Union[str, Path]) -> "LayeredConfig":
@@ -337,7 +398,7 @@ class LayeredConfig:
 
 
 # architecture name (config.json) -> "module:class" of the model that serves it
-ARCHITECTURES: Dict[str, str] = {"Bavesun": "lit_gpt.layered:LayeredGPT", "Rigulorn": "lit_gpt.layered:LayeredGPT"}
+ARCHITECTURES: Dict[str, str] = {name: "lit_gpt.layered:LayeredGPT" for name in ("Bavesun", "Rigulorn", "Ravelorn")}
 
 
 def load_config(checkpoint_dir: Union[str, Path]) -> Union[Config, LayeredConfig]:

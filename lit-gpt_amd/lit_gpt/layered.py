@@ -12,6 +12,10 @@ The design named by ``config.architecture`` fixes the layer's shape (``config.de
 * parallel — h = norm(x); x <- x + mixer(h) + ff(h); then the optional per-layer token input. The norm's weight is
   stored around zero (offset 1); every matrix that reads h is one row block of a single fused input projection;
   logits come from the embedding table itself (tied, unscaled) after the final norm.
+* post — the sublayers read the residual x itself and their OUTPUT is normed before it joins the residual with a
+  constant factor m: x <- x + m norm1(mixer(x)), then x <- x + m norm2(ff(x)) (layer norms with weight and bias).
+  A learned position vector joins the embedding; logits pass a tanh soft cap. The norm + residual add of a
+  sublayer is one launch that also leaves the bf16 copy of x the next input projection reads.
 * sequential — pre-norm sublayers, x <- x + mixer(norm1 x), then x <- x + ff(norm2 x) (a layer may have no
   feed-forward), over ``config.streams`` parallel residual streams: a sublayer reads a weighted sum of the streams
   and its output is written into all of them while a small matrix mixes them (``lit_gpt.mixers.StreamLinks``; one
@@ -157,6 +161,77 @@ class SequentialBlock(nn.Module):
         return [self.sub1] if self.sub2 is None else [self.sub1, self.sub2]
 
 
+class PostSublayer(nn.Module):
+    """One sublayer of a post-norm layer: the fused input projection of everything that reads the residual, the
+    module (a mixer or a feed-forward), and the layer norm (weight, bias) its output passes."""
+
+    def __init__(self, module: nn.Module, norm_w: torch.Tensor, norm_b: Optional[torch.Tensor], width: int, device,
+                 dtype) -> None:
+        super().__init__()
+        self.module = module
+        if norm_w.numel() != width or (norm_b is not None and norm_b.numel() != width):
+            raise ValueError("norm: weight and bias must have the model's width")
+        self.register_buffer("norm_w", norm_w.to(device=device, dtype=torch.float32).contiguous())
+        self.register_buffer("norm_b", None if norm_b is None else norm_b.to(device=device, dtype=torch.float32).contiguous())
+        w_in, offsets = _fuse_rows(module.in_parts(), width, device, dtype)
+        module.bind(offsets)
+        self.register_buffer("w_in", w_in)
+
+    def forward(self, x: torch.Tensor, x16: Optional[torch.Tensor], step: StepBatch, cache) -> torch.Tensor:
+        """x (T, width): the residual (x16: its bf16 copy for the MFMA tiles). Returns the sublayer's output, unnormed."""
+        n_in, W = self.w_in.shape
+        proj = torch.empty(step.T, n_in, dtype=torch.float32, device=x.device)
+        seq_ops.linear(x if x16 is None else x16, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
+        y = torch.empty(step.T, W, dtype=torch.float32, device=x.device)
+        if cache is None:
+            self.module(proj, x, y, h16=x16, accumulate=False)
+        else:
+            self.module(proj, step, cache, y, accumulate=False)
+        return y
+
+
+class PostNormBlock(nn.Module):
+    """x <- x + m norm1(mixer(x)), then x <- x + m norm2(ff(x)) when the layer has a feed-forward."""
+
+    def __init__(self, index: int, spec: LayerSpec, config: LayeredConfig, w: Dict[str, torch.Tensor], device,
+                 dtype) -> None:
+        super().__init__()
+        W, eps, design = config.width, config.norm_eps, config.design
+        if design.norm != "layer":
+            raise NotImplementedError("post-norm layers use layer norms")
+        self.mixer = MIXERS[spec.mixer.kind](spec.mixer, W, eps, _sub(w, "mix."), device, dtype)
+        self.sub1 = PostSublayer(self.mixer, w["norm1"], w.get("norm1.b"), W, device, dtype)
+        self.sub2 = None
+        if spec.mlp is not None:
+            if spec.mlp.kind != "moe" or design.moe != "scores":
+                raise NotImplementedError("post-norm layers serve the score-routed mixture of experts")
+            mlp = SparseFeedForward(spec.mlp, W, _sub(w, "mlp."), device, dtype, route="scores")
+            self.sub2 = PostSublayer(mlp, w["norm2"], w.get("norm2.b"), W, device, dtype)
+
+    def sublayers(self) -> List[PostSublayer]:
+        return [self.sub1] if self.sub2 is None else [self.sub1, self.sub2]
+
+
+def _mixer_shapes(p: str, m, W: int) -> Dict[str, Tuple[int, ...]]:
+    """Name -> shape of the tensors of a gated delta rule, a sink attention or a pair of them under prefix p."""
+    if m.kind == "parallel":
+        return {**_mixer_shapes(p + "left.", m.left, W), **_mixer_shapes(p + "right.", m.right, W)}
+    if m.kind == "sink_attention":
+        return {p + "q": (m.heads * m.dim, W), p + "k": (m.kv_heads * m.dim, W), p + "v": (m.kv_heads * m.vdim, W),
+                p + "sink": (m.heads,), p + "o": (W, m.heads * m.vdim)}
+    qk, v = m.kv_heads * m.dim, m.heads * m.vdim
+    out = {p + "q": (qk, W), p + "q.conv": (qk, m.conv), p + "k": (qk, W), p + "k.conv": (qk, m.conv), p + "v": (v, W),
+           p + "v.conv": (v, m.conv), p + "b": (m.heads, W), p + "A_log": (m.heads,), p + "norm": (m.vdim,),
+           p + "o": (W, v)}
+    if m.kind == "channel_delta":
+        ra, rg = m.decay_rank or 16, m.gate_rank or 16
+        out.update({p + "a1": (ra, W), p + "a2": (m.heads * m.dim, ra), p + "dt_bias": (m.heads * m.dim,),
+                    p + "g1": (rg, W), p + "g2": (v, rg)})
+    else:
+        out.update({p + "a": (m.heads, W), p + "dt_bias": (m.heads,), p + "g": (v, W)})
+    return out
+
+
 class LayeredGPT(nn.Module):
     decode_graph = False  # generate.base.generate steps this model eagerly (its graph executor is GPT's)
 
@@ -180,7 +255,19 @@ class LayeredGPT(nn.Module):
             self.side_embed = t.to(device=device, dtype=dtype).contiguous()
         design = config.design
         self.sequential = design.block == "sequential"
-        if self.sequential:
+        self.post = design.block == "post"
+        self.register_buffer("pos_table", None)
+        if design.positions == "learned":
+            t = weights["pos"]
+            if tuple(t.shape) != (config.max_positions, W):
+                raise ValueError(f"pos: shape {tuple(t.shape)}, expected {(config.max_positions, W)}")
+            self.pos_table = t.to(device=device, dtype=dtype).contiguous()
+        if self.post:
+            if config.side_dim or config.streams != 1:
+                raise NotImplementedError("post-norm layers have one residual stream and no per-layer token input")
+            self.blocks = nn.ModuleList(PostNormBlock(i, spec, config, _sub(weights, f"l{i}."), device, dtype)
+                                        for i, spec in enumerate(config.layers))
+        elif self.sequential:
             if config.side_dim:
                 raise NotImplementedError("per-layer token inputs belong to the parallel layers")
             self.blocks = nn.ModuleList(SequentialBlock(i, spec, config, _sub(weights, f"l{i}."), device, dtype)
@@ -197,8 +284,15 @@ class LayeredGPT(nn.Module):
             if tuple(weights["head"].shape) != (V, W):
                 raise ValueError(f"head: shape {tuple(weights['head'].shape)}, expected {(V, W)}")
             self.head = weights["head"].to(device=device, dtype=dtype).contiguous()
-        self.final_norm = StreamRMSNorm(W, eps=config.norm_eps, offset=design.norm_offset)
-        self.final_norm.weight = weights["final.norm"].to(device=device, dtype=torch.float32).contiguous()
+        self.register_buffer("final_bias", None)
+        if design.norm == "layer":
+            self.final_norm = None
+            self.register_buffer("final_weight", weights["final.norm"].to(device=device, dtype=torch.float32).contiguous())
+            if "final.norm.b" in weights:
+                self.final_bias = weights["final.norm.b"].to(device=device, dtype=torch.float32).contiguous()
+        else:
+            self.final_norm = StreamRMSNorm(W, eps=config.norm_eps, offset=design.norm_offset)
+            self.final_norm.weight = weights["final.norm"].to(device=device, dtype=torch.float32).contiguous()
         self.runs: List[int] = config.layer_runs
         self.caches: Optional[nn.ModuleList] = None  # one cache / state per layer run
         self._max_seq_length = 0
@@ -222,11 +316,18 @@ class LayeredGPT(nn.Module):
             out["head"] = (config.vocab, config.width)
         if config.side_dim:
             out["side.embed"] = (config.vocab, config.side_dim * len(config.layers))
+        biased = config.design.norm == "layer"
+        if biased:
+            out["final.norm.b"] = (W,)
+        if config.design.positions == "learned":
+            out["pos"] = (config.max_positions, W)
         for i, spec in enumerate(config.layers):
             m, p = spec.mixer, f"l{i}."
             out[p + "norm1"] = (W,)
-            if spec.mlp is not None and config.design.block == "sequential":
+            if spec.mlp is not None and config.design.block != "parallel":
                 out[p + "norm2"] = (W,)
+            if biased:
+                out.update({name + ".b": (W,) for name in (p + "norm1", p + "norm2") if name in out})
             if config.stream_weights:
                 for q in (1, 2) if spec.mlp is not None else (1,):
                     s = config.streams
@@ -240,6 +341,8 @@ class LayeredGPT(nn.Module):
                 if m.kv_from is None:
                     out.update({p + "mix.k": (2 * m.kv_heads * m.dim, W), p + "mix.v": (m.kv_heads * m.vdim, W)})
                 out.update({p + f"mix.{n}": (m.dim,) for n in ("lq1", "lk1", "lq2", "lk2")})
+            elif m.kind in ("channel_delta", "gated_delta", "sink_attention", "parallel"):
+                out.update(_mixer_shapes(p + "mix.", m, W))
             elif m.kind == "mamba2":
                 inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
                 out.update({p + "mix.in": (2 * inner + bc + m.heads, W), p + "mix.conv": (inner + bc, m.conv),
@@ -254,8 +357,13 @@ class LayeredGPT(nn.Module):
             if f is not None and f.kind == "dense":
                 out.update({p + "mlp.gate": (f.ff, W), p + "mlp.up": (f.ff, W), p + "mlp.down": (W, f.ff)})
             elif f is not None:
-                out[p + "mlp.router"] = (f.experts, W)
+                gated = config.design.moe == "scores"
+                out[p + "mlp.router"] = (f.experts + (f.identity if gated else 0), W)
+                if gated:
+                    out[p + "mlp.correction"] = (f.experts + f.identity,)
                 for e in range(f.experts):
+                    if gated:
+                        out[p + f"mlp.e{e}.gate"] = (f.ff, W)
                     out.update({p + f"mlp.e{e}.up": (f.ff, W), p + f"mlp.e{e}.down": (W, f.ff)})
             if config.side_dim:
                 out.update({p + "side.gate": (config.side_dim, W), p + "side.proj": (W, config.side_dim),
@@ -273,6 +381,13 @@ class LayeredGPT(nn.Module):
             leaf = name.rsplit(".", 1)[-1]
             if leaf in ("norm1", "norm2") or name == "final.norm":
                 t = neutral + 0.1 * torch.randn(shape, generator=g)
+            elif name.endswith(("norm1.b", "norm2.b", "final.norm.b", "correction")):
+                t = 0.1 * torch.randn(shape, generator=g)
+            elif name == "pos":
+                t = 0.5 * shape[1] ** -0.5 * torch.randn(shape, generator=g)
+            elif name.endswith(".conv") and len(shape) == 2 and ".mix." in name and "mamba" not in name and \
+                    name.rsplit(".", 2)[-2] in ("q", "k", "v"):
+                t = torch.randn(shape, generator=g) * 0.7
             elif ".hc" in name:
                 s = config.streams
                 t = {"in": torch.full(shape, 1.0 / s), "out": torch.ones(shape), "mix": torch.eye(s)}[leaf] + \
@@ -305,6 +420,8 @@ class LayeredGPT(nn.Module):
 
     @max_seq_length.setter
     def max_seq_length(self, value: int) -> None:
+        if self.config.max_positions > 0:  # a learned position table bounds every sequence
+            value = min(int(value), self.config.max_positions)
         if self.caches is not None and value != self._max_seq_length:
             self.caches = None  # rebuilt by the next set_kv_cache
         self._max_seq_length = int(value)
@@ -348,9 +465,30 @@ class LayeredGPT(nn.Module):
             raise TypeError("You need to call `set_kv_cache()`")
         if self.sequential:
             return self._forward_streams(step)
+        if self.post:
+            return self._forward_post(step)
         x = seq_ops.embed(step.tokens, self.embed, self.config.embedding_scale)
         for run, layer in enumerate(self.runs):
             self.blocks[layer](x, step, self.caches[run])
+        return x
+
+    def _forward_post(self, step: StepBatch, after_layer=None) -> torch.Tensor:
+        """The post-norm layers: every sublayer reads the residual itself (for more than 8 rows with bf16 weights its
+        bf16 copy, which the embedding and every norm + residual launch leave behind); its output passes the layer
+        norm and joins the residual times ``residual_mult`` in one launch. ``after_layer(run, x)``: a hook that sees
+        the residual (T, width) after each layer run (for tests)."""
+        cfg = self.config
+        want16 = step.T > 8 and self.dtype == torch.bfloat16
+        got = seq_ops.embed_pos(step.tokens, step.pos, self.embed, self.pos_table, cfg.embedding_scale, bf16_copy=want16)
+        x, x16 = got if want16 else (got, None)
+        for run, layer in enumerate(self.runs):
+            for k, sub in enumerate(self.blocks[layer].sublayers()):
+                y = sub(x, x16, step, self.caches[run] if k == 0 else None)
+                got = seq_ops.layernorm(y, sub.norm_w, sub.norm_b, eps=cfg.norm_eps, x=x, mult=cfg.residual_mult,
+                                        bf16_copy=want16)
+                x16 = got[1] if want16 else None
+            if after_layer is not None:
+                after_layer(run, x)
         return x
 
     def _forward_streams(self, step: StepBatch, after_layer=None) -> torch.Tensor:
@@ -386,11 +524,17 @@ class LayeredGPT(nn.Module):
         rows of the stream (int32 indices; all if None)."""
         if rows is not None:
             x = seq_ops.gather_rows(x, rows)
-        h = self.final_norm(x)
+        if self.final_norm is None:
+            h = seq_ops.layernorm(x, self.final_weight, self.final_bias, eps=self.config.norm_eps)
+        else:
+            h = self.final_norm(x)
         table = self.embed if self.head is None else self.head
         V, W = table.shape
         out = torch.empty(h.shape[0], V, dtype=torch.float32, device=h.device)
-        return seq_ops.linear(h, table, M=h.shape[0], N=V, K=W, y=out, lda=W, ldy=V)
+        seq_ops.linear(h, table, M=h.shape[0], N=V, K=W, y=out, lda=W, ldy=V)
+        if self.config.logit_softcap > 0.0:
+            seq_ops.softcap(out, self.config.logit_softcap)
+        return out
 
     def forward(self, idx: torch.Tensor, input_pos: Optional[torch.Tensor] = None, *,
                 last_token_only: bool = False) -> torch.Tensor:

@@ -22,7 +22,7 @@ import torch.nn as nn
 
 from lit_gpt import seq_ops
 from lit_gpt.config import FeedForwardSpec, MixerSpec
-from lit_gpt.model import HeadKVCache, LatentKVCache, RetentionState, ScanState
+from lit_gpt.model import CachePair, HeadKVCache, LatentKVCache, RetentionState, ScanState
 
 
 @dataclass
@@ -275,6 +275,150 @@ class SelectiveScan(InputReader):
         seq_ops.linear(g, self.w_o, M=step.T, N=W, K=inner, y=x, lda=inner, ldy=W, accumulate=accumulate)
 
 
+class GatedDelta(InputReader):
+    """The gated delta rule: per head an outer-product memory S (dim x vdim, fp32) that is decayed, corrected towards
+    the current key's value and read by the query: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
+    q and k (``kv_heads`` heads shared by groups of value heads) and v pass a short causal per-channel convolution
+    (tap ``taps - 1`` weights the token itself, no bias) and silu; q and k become unit vectors per head
+    (x / sqrt(sum x^2 + 1e-6)), q also times dim^-1/2; beta = sigmoid(W_b h); g = exp(-exp(A_log) softplus(a + dt_bias)).
+    ``per_channel``: a = W_a2 (W_a1 h) with one decay per head and key channel and the output gate is
+    sigmoid(W_g2 (W_g1 h)); otherwise a = W_a h with one decay per head and the gate is silu(W_g h). Each head's output
+    is divided by its root mean square, times a weight shared by the heads, times the gate, then projected. The state
+    (S and the convolution's last taps - 1 inputs) lives in a cache slot."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype,
+                 per_channel: Optional[bool] = None) -> None:
+        super().__init__()
+        self.H, self.G, self.d, self.dv, self.taps, self.eps = spec.heads, spec.kv_heads, spec.dim, spec.vdim, spec.conv, eps
+        self.per_channel = spec.kind == "channel_delta" if per_channel is None else per_channel
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        self.channels = 2 * G * d + H * dv
+        shapes = [("q", (G * d, width)), ("k", (G * d, width)), ("v", (H * dv, width)), ("q.conv", (G * d, self.taps)),
+                  ("k.conv", (G * d, self.taps)), ("v.conv", (H * dv, self.taps)), ("b", (H, width)), ("A_log", (H,)),
+                  ("norm", (dv,)), ("o", (width, H * dv))]
+        if self.per_channel:
+            ra, rg = w["a1"].shape[0], w["g1"].shape[0]
+            shapes += [("a1", (ra, width)), ("a2", (H * d, ra)), ("g1", (rg, width)), ("g2", (H * dv, rg)),
+                       ("dt_bias", (H * d,))]
+        else:
+            shapes += [("a", (H, width)), ("g", (H * dv, width)), ("dt_bias", (H,))]
+        for name, shape in shapes:
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"{spec.kind}.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        self._in = [("qkv", torch.cat([w["q"], w["k"], w["v"]])), ("b", w["b"])]
+        self._in += [("a1", w["a1"]), ("g1", w["g1"])] if self.per_channel else [("a", w["a"]), ("g", w["g"])]
+        if self.per_channel:
+            self.register_buffer("w_a2", w["a2"].to(device=device, dtype=dtype).contiguous())
+            self.register_buffer("w_g2", w["g2"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("conv_w", torch.cat([w["q.conv"], w["k.conv"], w["v.conv"]]).to(device=device, dtype=dtype)
+                             .contiguous())
+        self.register_buffer("conv_b", torch.zeros(self.channels, device=device, dtype=dtype))
+        for name, key in (("A_log", "A_log"), ("dt_bias", "dt_bias"), ("norm_w", "norm")):
+            self.register_buffer(name, _f32(w[key], device))
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> ScanState:
+        return ScanState(slots, self.H, self.d, self.dv, self.taps, self.channels, device=device)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: ScanState, x: torch.Tensor, accumulate: bool = True,
+                post: float = 1.0) -> None:
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        T, ld = proj.shape
+        tables = (step.seq_start, step.seq_slot, step.seq_pos0)
+        qkv = seq_ops.conv_silu(proj, self.off["qkv"], self.conv_w, self.conv_b, cache.conv, *tables,
+                                step.max_len or T)
+        if self.per_channel:
+            ra, rg = self.w_a2.shape[1], self.w_g2.shape[1]
+            a = torch.empty(T, H * d, dtype=torch.float32, device=proj.device)
+            seq_ops.linear(proj, self.w_a2, M=T, N=H * d, K=ra, y=a, a_off=self.off["a1"], lda=ld, ldy=H * d)
+            gate = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
+            seq_ops.linear(proj, self.w_g2, M=T, N=H * dv, K=rg, y=gate, a_off=self.off["g1"], lda=ld, ldy=H * dv)
+            a_off, g_off, act = 0, 0, seq_ops.ACT_SIGMOID
+        else:
+            a, a_off, gate, g_off, act = proj, self.off["a"], proj, self.off["g"], seq_ops.ACT_SILU
+        dec, beta = seq_ops.delta_prepare(qkv, a, a_off, proj, self.off["b"], self.A_log, self.dt_bias, H=H, G=G, d=d,
+                                          per_channel=self.per_channel, q_scale=float(d) ** -0.5)
+        o = seq_ops.gated_delta(qkv, dec, beta, cache.s, *tables, H=H, G=G, d=d, dv=dv, per_channel=self.per_channel)
+        o = seq_ops.head_gate(o, gate, g_off, H=H, dv=dv, unit_norm=True, eps=self.eps, act=act, weight=self.norm_w,
+                              post=post, bf16_copy=_tiles16(T, self.w_o))
+        W = x.shape[1]
+        seq_ops.linear(o, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
+
+
+class SinkAttention(InputReader):
+    """Causal softmax attention with grouped key / value heads and no rotation: q and k are divided by their root
+    mean square per head (no weight), the query is multiplied by a temperature that grows with its position,
+    1 + coef * ln(floor((p + 1) / every) + 1); score = (q . k) * scale; a learned per-head sink scalar adds its
+    exponential to the softmax normaliser without contributing a value. The cache holds the normed keys and the
+    values."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        self.H, self.G, self.d, self.dv, self.eps = spec.heads, spec.kv_heads, spec.dim, spec.vdim, eps
+        self.scale, self.cap, self.chunk = spec.scale, spec.softcap, spec.mask_size
+        self.temp_coef, self.temp_every = spec.q_temp_coef, spec.q_temp_every
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        for name, shape in (("q", (H * d, width)), ("k", (G * d, width)), ("v", (G * dv, width)), ("o", (width, H * dv))):
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"sink_attention.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        if "sink" in w and w["sink"].numel() != H:
+            raise ValueError(f"sink_attention.sink: {w['sink'].numel()} values, expected {H}")
+        self._in = [(n, w[n]) for n in ("q", "k", "v")]
+        self.register_buffer("sink", _f32(w["sink"], device) if "sink" in w else None)
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> HeadKVCache:
+        return HeadKVCache(slots, max_seq_length, self.G, self.d, self.dv, device=device, dtype=dtype)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: HeadKVCache, x: torch.Tensor, accumulate: bool = True,
+                post: float = 1.0) -> None:
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        seq_ops.normattn_prepare(proj, self.off["q"], self.off["k"], self.off["v"], cache.k, cache.v, step.slot,
+                                 step.pos, H=H, G=G, d=d, dv=dv, eps=self.eps, temp_coef=self.temp_coef,
+                                 temp_every=self.temp_every)
+        att = seq_ops.sinkattn(proj, self.off["q"], cache.k, cache.v, self.sink, step.seq_start, step.seq_slot,
+                               step.seq_pos0, step.max_len or step.T, H=H, G=G, d=d, dv=dv, scale=self.scale,
+                               chunk=self.chunk, cap=self.cap, post=post, bf16_copy=_tiles16(step.T, self.w_o))
+        W = x.shape[1]
+        seq_ops.linear(att, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
+
+
+class ParallelMixer(InputReader):
+    """Two mixers side by side on the same input, summed with fixed factors: ``left_scale`` * a sink attention
+    (tensors under ``left.``) + ``right_scale`` * a gated delta rule with one decay per head (``right.``). Both read
+    the layer's one input projection; each factor is applied where its mixer's last elementwise kernel runs, and the
+    second out-projection accumulates onto the first."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        sub = lambda prefix: {k[len(prefix):]: v for k, v in w.items() if k.startswith(prefix)}  # noqa: E731
+        self.left = SinkAttention(spec.left, width, eps, sub("left."), device, dtype)
+        self.right = GatedDelta(spec.right, width, eps, sub("right."), device, dtype, per_channel=False)
+        self.left_scale, self.right_scale = spec.left_scale, spec.right_scale
+
+    def in_parts(self):
+        return [("left." + n, t) for n, t in self.left.in_parts()] + [("right." + n, t) for n, t in self.right.in_parts()]
+
+    def bind(self, offsets: Dict[str, int]) -> None:
+        self.left.bind({k[5:]: v for k, v in offsets.items() if k.startswith("left.")})
+        self.right.bind({k[6:]: v for k, v in offsets.items() if k.startswith("right.")})
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> CachePair:
+        return CachePair(self.left.build_cache(slots, max_seq_length, device, dtype),
+                         self.right.build_cache(slots, max_seq_length, device, dtype))
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: CachePair, x: torch.Tensor,
+                accumulate: bool = True) -> None:
+        self.left(proj, step, cache.left, x, accumulate=accumulate, post=self.left_scale)
+        self.right(proj, step, cache.right, x, accumulate=True, post=self.right_scale)
+
+
 class StreamLinks(nn.Module):
     """The weights that tie one sublayer to a multi-stream residual: ``read`` (s,) weights of the sum the sublayer
     reads, ``write`` (s,) weights of its output in every stream, ``mix`` (s, s) [from, to] applied to the streams
@@ -325,8 +469,14 @@ class GatedFeedForward(InputReader):
 
 
 class SparseFeedForward(InputReader):
-    """Mixture of experts: fp32 router logits, the ``top`` largest selected, weights = softmax restricted to the selected
-    logits, expert = W_down act(W_up h) without biases (``act`` defaults to the square of relu).
+    """Mixture of experts with an fp32 router, in one of two forms.
+
+    ``route = "top_logits"``: the ``top`` largest logits are chosen, weights = softmax restricted to the chosen
+    logits, expert = W_down act(W_up h) (``act`` defaults to the square of relu).
+    ``route = "scores"``: scores = softmax over ALL router outputs; the ``top`` largest of score + ``correction``
+    (a stored vector that shifts the choice only) are chosen; the weights are the chosen scores as they are;
+    expert = W_down (act(W_gate h) * W_up h) (``act`` defaults to silu); the last ``identity`` router outputs are
+    identity experts without matrices, whose output is the input itself.
 
     Few (token, choice) pairs (decode) stream only the chosen experts' rows through two GEMV launches. A prompt
     sorts its pairs by expert on the device and runs two grouped products over the expert ranges, then sums each
@@ -335,41 +485,64 @@ class SparseFeedForward(InputReader):
     STREAM_PAIRS = 48  # up to this many (token, choice) pairs the streaming form runs
 
     def __init__(self, spec: FeedForwardSpec, width: int, w: Dict[str, torch.Tensor], device, dtype,
-                 act: int = seq_ops.ACT_RELU2) -> None:
+                 act: Optional[int] = None, route: str = "top_logits") -> None:
         super().__init__()
-        self.E, self.top, self.ff, self.act = spec.experts, spec.top, spec.ff, act
-        if tuple(w["router"].shape) != (spec.experts, width):
-            raise ValueError(f"mlp.router: shape {tuple(w['router'].shape)}, expected {(spec.experts, width)}")
+        if route not in ("top_logits", "scores"):
+            raise ValueError(f"unknown routing {route!r}")
+        self.E, self.top, self.ff, self.route = spec.experts, spec.top, spec.ff, route
+        self.gated = route == "scores"
+        self.n_router = spec.experts + (spec.identity if self.gated else 0)
+        self.act = act if act is not None else (seq_ops.ACT_SILU if self.gated else seq_ops.ACT_RELU2)
+        if tuple(w["router"].shape) != (self.n_router, width):
+            raise ValueError(f"mlp.router: shape {tuple(w['router'].shape)}, expected {(self.n_router, width)}")
         self._in = [("router", w["router"])]
-        up = torch.stack([w[f"e{e}.up"] for e in range(self.E)])
+        up = torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) if self.gated else w[f"e{e}.up"]
+                          for e in range(self.E)])
         down = torch.stack([w[f"e{e}.down"] for e in range(self.E)])
-        if tuple(up.shape) != (self.E, spec.ff, width) or tuple(down.shape) != (self.E, width, spec.ff):
+        rows = 2 * spec.ff if self.gated else spec.ff
+        if tuple(up.shape) != (self.E, rows, width) or tuple(down.shape) != (self.E, width, spec.ff):
             raise ValueError("mlp experts: unexpected shapes")
-        self.register_buffer("w_up", up.to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("w_up", up.to(device=device, dtype=dtype).contiguous())  # gated: gate rows, then up rows
         self.register_buffer("w_down", down.to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("correction", None)
+        if self.gated and "correction" in w:
+            if w["correction"].numel() != self.n_router:
+                raise ValueError(f"mlp.correction: {w['correction'].numel()} values, expected {self.n_router}")
+            self.correction = _f32(w["correction"], device)
 
     def in_parts(self):
         return self._in
 
-    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor,
-                h16: Optional[torch.Tensor] = None) -> None:
-        """h: the norm output (fp32); h16: its bf16 copy when the layer made one (the grouped products read it)."""
+    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor, h16: Optional[torch.Tensor] = None,
+                accumulate: bool = True) -> None:
+        """h: the sublayer's input (fp32); h16: its bf16 copy when the layer made one (the grouped products read it)."""
         T, W = h.shape
         E, top, F = self.E, self.top, self.ff
-        ids, wts = seq_ops.moe_route(proj, self.off["router"], E, top)
+        if self.gated:
+            ids, wts = seq_ops.moe_route_scores(proj, self.off["router"], self.n_router, top, self.correction)
+        else:
+            ids, wts = seq_ops.moe_route(proj, self.off["router"], E, top)
         if T * top <= self.STREAM_PAIRS:
-            a = seq_ops.moe_up(h, self.w_up, ids, self.act)
-            seq_ops.moe_down(a, self.w_down, ids, wts, x)
+            a = seq_ops.moe_up(h, self.w_up, ids, self.act, gated=self.gated)
+            seq_ops.moe_down(a, self.w_down, ids, wts, x, h, accumulate=accumulate)
             return
         pairs = T * top
-        z_start, tok_of, where = seq_ops.moe_sort(ids, E)
-        a = torch.empty(pairs, F, dtype=torch.bfloat16 if self.w_down.dtype == torch.bfloat16 else torch.float32,
-                        device=h.device)
-        seq_ops.linear(h if h16 is None else h16, self.w_up, M=pairs, N=F, K=W, y=a, lda=W, ldy=F, batch=E,
-                       stride_w=F * W, act=self.act, a_rows=tok_of, z_start=z_start)
+        z_start, tok_of, where = seq_ops.moe_sort(ids, self.n_router)
+        a_dtype = torch.bfloat16 if self.w_down.dtype == torch.bfloat16 else torch.float32
+        if self.gated:
+            gu = torch.empty(pairs, 2 * F, dtype=torch.float32, device=h.device)
+            seq_ops.linear(h if h16 is None else h16, self.w_up, M=pairs, N=2 * F, K=W, y=gu, lda=W, ldy=2 * F, batch=E,
+                           stride_w=2 * F * W, a_rows=tok_of, z_start=z_start)
+            a = seq_ops.glu(gu, 0, F, F, self.act, bf16=a_dtype == torch.bfloat16)
+        else:
+            a = torch.empty(pairs, F, dtype=a_dtype, device=h.device)
+            seq_ops.linear(h if h16 is None else h16, self.w_up, M=pairs, N=F, K=W, y=a, lda=W, ldy=F, batch=E,
+                           stride_w=F * W, act=self.act, a_rows=tok_of, z_start=z_start)
         y = torch.empty(pairs, W, dtype=torch.float32, device=h.device)
         seq_ops.linear(a, self.w_down, M=pairs, N=W, K=F, y=y, lda=F, ldy=W, batch=E, stride_w=W * F, z_start=z_start)
-        seq_ops.moe_combine(y, where, wts, x)
+        identity = self.n_router > E
+        seq_ops.moe_combine(y, where, wts, x, ids=ids if identity else None, n_real=E, h=h if identity else None,
+                            accumulate=accumulate)
 
 
 class TokenSide(nn.Module):
@@ -391,4 +564,5 @@ class TokenSide(nn.Module):
 
 
 MIXERS = {"retention": Retention, "latent_attention": LatentAttention, "attention": DiffAttention,
-          "mamba2": SelectiveScan}
+          "mamba2": SelectiveScan, "channel_delta": GatedDelta, "gated_delta": GatedDelta,
+          "sink_attention": SinkAttention, "parallel": ParallelMixer}

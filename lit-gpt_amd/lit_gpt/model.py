@@ -731,6 +731,27 @@ class ScanState(nn.Module):
         torch.nn.init.zeros_(self.conv)
 
 
+class CachePair(nn.Module):
+    """The caches of two mixers that run side by side in one layer (``left`` and ``right``), handed out, grown and
+    cleared together."""
+
+    def __init__(self, left: nn.Module, right: nn.Module) -> None:
+        super().__init__()
+        self.left, self.right = left, right
+
+    @property
+    def slots(self) -> int:
+        return self.left.slots
+
+    def grow(self, slots: int) -> None:
+        self.left.grow(slots)
+        self.right.grow(slots)
+
+    def reset_parameters(self) -> None:
+        self.left.reset_parameters()
+        self.right.reset_parameters()
+
+
 def build_rope_cache(seq_len: int, n_elem: int, device: Optional[torch.device] = None, base: int = 10000,
                      condense_ratio: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
     """cos/sin tables (seq_len, n_elem) in fp32 (model.py:746-764).

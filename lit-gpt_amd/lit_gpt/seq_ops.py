@@ -36,16 +36,17 @@ SIGNATURES = {
     "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P, _P],
     "lgs_gather_rows": [_P, _P, _P, _I, _I, _P],
     "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _P],
-    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P, _P],
+    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P, _F, _P, _P],
     "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
     "lgs_latent_attention_tiles": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _I, _P],
     "lgs_moe_route": [_P, _L, _I, _I, _I, _P, _P, _P],
-    "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
-    "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _P],
+    "lgs_moe_route_scores": [_P, _L, _I, _I, _I, _P, _P, _P, _P],
+    "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _L, _I, _P],
     "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
-    "lgs_moe_combine": [_P, _P, _P, _P, _L, _I, _I, _I, _P],
+    "lgs_moe_combine": [_P, _P, _P, _P, _L, _I, _I, _I, _P, _I, _P, _L, _I, _P],
     "lgs_token_side": [_P, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],
     "lgs_embed_streams": [_P, _P, _I, _F, _P, _I, _I, _I, _I, _P],
     "lgs_streams_step": [_P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _P],
@@ -56,6 +57,13 @@ SIGNATURES = {
     "lgs_ssm_scan": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
     "lgs_gated_group_norm": [_P, _P, _L, _P, _F, _P, _P, _I, _I, _I, _P],
     "lgs_glu_clamped": [_P, _P, _L, _P, _I, _I, _I, _F, _F, _F, _P],
+    "lgs_embed_pos": [_P, _P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],
+    "lgs_layernorm": [_P, _P, _P, _F, _F, _I, _P, _P, _I, _I, _P],
+    "lgs_softcap": [_P, _L, _F, _P],
+    "lgs_normattn_prepare": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P],
+    "lgs_sinkattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P],
+    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
+    "lgs_gated_delta": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
 }
 _RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
 
@@ -213,16 +221,18 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: tor
 
 
 def head_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, *, H: int, dv: int, unit_norm: bool, eps: float,
-              act: int, bf16_copy: bool = False) -> torch.Tensor:
-    """In place on o (T, H * dv): per head optional unit RMS, then times act(gate), the gate at proj[:, g_off:].
-    Returns o, or with ``bf16_copy`` its rounding to bf16 (the operand of a bf16 MFMA product)."""
+              act: int, bf16_copy: bool = False, weight: Optional[torch.Tensor] = None,
+              post: float = 1.0) -> torch.Tensor:
+    """In place on o (T, H * dv): per head optional unit RMS, times ``weight`` (dv values shared by the heads), times
+    act(gate), the gate at proj[:, g_off:], times ``post``. Returns o, or with ``bf16_copy`` its rounding to bf16
+    (the operand of a bf16 MFMA product)."""
     T, ld = proj.shape
-    if o.shape != (T, H * dv) or g_off + H * dv > ld:
+    if o.shape != (T, H * dv) or g_off + H * dv > ld or (weight is not None and weight.numel() != dv):
         raise ValueError("head_gate: shapes")
     o16 = torch.empty(T, H * dv, dtype=torch.bfloat16, device=o.device) if bf16_copy else None
     _check(load_library().lgs_head_gate(_dev(o, "o", F32), _dev(proj, "proj", F32) + 4 * g_off, ld, T, H, dv,
-                                        int(unit_norm), float(eps), act, _opt(o16, "o_bf16", torch.bfloat16),
-                                        _stream()))
+                                        int(unit_norm), float(eps), act, _opt(weight, "weight", F32), float(post),
+                                        _opt(o16, "o_bf16", torch.bfloat16), _stream()))
     return o16 if bf16_copy else o
 
 
@@ -307,26 +317,46 @@ def moe_route(proj: torch.Tensor, z_off: int, E: int, top: int):
     return ids, wts
 
 
-def moe_up(h: torch.Tensor, up: torch.Tensor, ids: torch.Tensor, act: int) -> torch.Tensor:
+def moe_route_scores(proj: torch.Tensor, z_off: int, E: int, top: int, bias: Optional[torch.Tensor] = None):
+    """Softmax over all E router outputs at proj[:, z_off:]; the ``top`` largest of score + ``bias`` are chosen
+    (lowest index first among equals); the weights are the chosen scores themselves, not renormalised."""
+    T, ld = proj.shape
+    if z_off + E > ld or (bias is not None and bias.numel() != E):
+        raise ValueError("moe_route_scores: router logits outside the row, or the correction's size")
+    ids = torch.empty(T, top, dtype=I32, device=proj.device)
+    wts = torch.empty(T, top, dtype=F32, device=proj.device)
+    _check(load_library().lgs_moe_route_scores(_dev(proj, "proj", F32) + 4 * z_off, ld, T, E, top,
+                                               _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), _stream()))
+    return ids, wts
+
+
+def moe_up(h: torch.Tensor, up: torch.Tensor, ids: torch.Tensor, act: int, gated: bool = False) -> torch.Tensor:
+    """up (E, F, K), or with ``gated`` (E, 2 F, K): F gate rows, then F up rows -> act(gate h) * (up h). Pairs whose
+    expert id is >= E (experts without matrices) are left untouched."""
     T, K = h.shape
     E, F, K2 = up.shape
+    if gated:
+        F //= 2
     top = ids.shape[1]
     if K2 != K or ids.shape[0] != T:
         raise ValueError("moe_up: shapes")
     buf = torch.empty(T * top, F, dtype=F32, device=h.device)
     _check(load_library().lgs_moe_up(_dev(h, "h", F32), K, _dev(up, "up"), _wf32(up, "up"), _dev(ids, "ids", I32),
-                                     buf.data_ptr(), T, top, F, K, act, _stream()))
+                                     buf.data_ptr(), T, top, F, K, act, int(gated), E, _stream()))
     return buf
 
 
-def moe_down(actbuf: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, x: torch.Tensor) -> None:
+def moe_down(actbuf: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, x: torch.Tensor,
+             h: torch.Tensor, accumulate: bool = True) -> None:
+    """x (+)= sum over a token's choices of weight * down[expert] act; a choice whose id is >= the number of stored
+    experts is an identity expert and contributes weight * h."""
     T, top = ids.shape
     E, N, F = down.shape
-    if actbuf.shape != (T * top, F) or x.shape != (T, N):
+    if actbuf.shape != (T * top, F) or x.shape != (T, N) or h.shape != (T, N):
         raise ValueError("moe_down: shapes")
     _check(load_library().lgs_moe_down(_dev(actbuf, "actbuf", F32), _dev(down, "down"), _wf32(down, "down"),
                                        _dev(ids, "ids", I32), _dev(wts, "wts", F32), _dev(x, "x", F32), N, T, top, N,
-                                       F, _stream()))
+                                       F, E, _dev(h, "h", F32), N, int(accumulate), _stream()))
 
 
 def moe_sort(ids: torch.Tensor, E: int):
@@ -341,13 +371,18 @@ def moe_sort(ids: torch.Tensor, E: int):
     return z_start, tok_of, where
 
 
-def moe_combine(y: torch.Tensor, where: torch.Tensor, wts: torch.Tensor, x: torch.Tensor) -> None:
+def moe_combine(y: torch.Tensor, where: torch.Tensor, wts: torch.Tensor, x: torch.Tensor, *,
+                ids: Optional[torch.Tensor] = None, n_real: int = 0, h: Optional[torch.Tensor] = None,
+                accumulate: bool = True) -> None:
+    """x (+)= sum_k wts[:, k] * y[where[:, k]]; with ``ids`` a choice whose id is >= ``n_real`` (an identity expert)
+    contributes the token's input ``h`` instead."""
     T, top = wts.shape
     N = x.shape[1]
-    if y.shape != (T * top, N) or where.numel() != T * top:
+    if y.shape != (T * top, N) or where.numel() != T * top or (ids is not None and (h is None or h.shape != (T, N))):
         raise ValueError("moe_combine: shapes")
     _check(load_library().lgs_moe_combine(_dev(y, "y", F32), _dev(where, "where", I32), _dev(wts, "wts", F32),
-                                          _dev(x, "x", F32), N, T, top, N, _stream()))
+                                          _dev(x, "x", F32), N, T, top, N, _opt(ids, "ids", I32), int(n_real),
+                                          _opt(h, "h", F32), N, int(accumulate), _stream()))
 
 
 def token_side(x: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col0: int, gate_w: torch.Tensor,
@@ -529,4 +564,133 @@ def glu_clamped(proj: torch.Tensor, a_off: int, b_off: int, n: int, *, alpha: fl
     base = _dev(proj, "proj", F32)
     _check(load_library().lgs_glu_clamped(base + 4 * a_off, base + 4 * b_off, ld, out.data_ptr(), int(bf16), T, n,
                                           float(alpha), float(limit), float(shift), _stream()))
+    return out
+
+
+def embed_pos(tokens: torch.Tensor, pos: torch.Tensor, table: torch.Tensor, pos_table: torch.Tensor, scale: float,
+              bf16_copy: bool = False):
+    """x[t] = table[tokens[t]] * scale + pos_table[pos[t]] (T, W) fp32; with ``bf16_copy`` also its rounding."""
+    T, (V, W) = tokens.numel(), table.shape
+    if pos.numel() != T or pos_table.shape[1] != W or pos_table.dtype != table.dtype:
+        raise ValueError("embed_pos: shapes")
+    x = torch.empty(T, W, dtype=F32, device=tokens.device)
+    x16 = torch.empty(T, W, dtype=torch.bfloat16, device=tokens.device) if bf16_copy else None
+    _check(load_library().lgs_embed_pos(_dev(tokens, "tokens", I32), _dev(pos, "pos", I32), _dev(table, "table"),
+                                        _dev(pos_table, "pos_table"), _wf32(table, "table"), float(scale),
+                                        x.data_ptr(), _opt(x16, "x_bf16", torch.bfloat16), T, W, V,
+                                        pos_table.shape[0], _stream()))
+    return (x, x16) if bf16_copy else x
+
+
+def layernorm(y: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], *, eps: float,
+              x: Optional[torch.Tensor] = None, mult: float = 1.0, bf16_copy: bool = False):
+    """Layer norm of the rows of y (rows, n): (y - mean) / sqrt(var + eps) * weight + bias, var the mean of the squared
+    deviations. With ``x`` the result joins a residual in place, x += mult * norm (a sublayer's normed output);
+    without, it is returned times ``mult``. ``bf16_copy``: also the rounding of the result (of the new x) to bf16."""
+    rows, n = y.shape
+    if weight.numel() != n or (bias is not None and bias.numel() != n) or (x is not None and x.shape != y.shape):
+        raise ValueError("layernorm: shapes")
+    out = x if x is not None else torch.empty_like(y)
+    o16 = torch.empty(rows, n, dtype=torch.bfloat16, device=y.device) if bf16_copy else None
+    _check(load_library().lgs_layernorm(_dev(y, "y", F32), _dev(weight, "weight", F32), _opt(bias, "bias", F32),
+                                        float(eps), float(mult), int(x is not None), _dev(out, "x", F32),
+                                        _opt(o16, "x_bf16", torch.bfloat16), rows, n, _stream()))
+    return (out, o16) if bf16_copy else out
+
+
+def softcap(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """In place: cap * tanh(z / cap)."""
+    _check(load_library().lgs_softcap(_dev(z, "z", F32), z.numel(), float(cap), _stream()))
+    return z
+
+
+def normattn_prepare(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, cache_k: torch.Tensor,
+                     cache_v: torch.Tensor, slot: torch.Tensor, pos: torch.Tensor, *, H: int, G: int, d: int, dv: int,
+                     eps: float, temp_coef: float = 0.0, temp_every: int = 0) -> None:
+    """Unit-RMS queries (times the position's query temperature) in place in ``proj``; unit-RMS keys and the values
+    into the cache rows (slot, position). cache_k (slots, S, G, d), cache_v (slots, S, G, dv)."""
+    T, ld = proj.shape
+    slots, S = cache_k.shape[:2]
+    if tuple(cache_k.shape) != (slots, S, G, d) or tuple(cache_v.shape) != (slots, S, G, dv) or \
+            cache_k.dtype != cache_v.dtype:
+        raise ValueError("normattn_prepare: cache shapes")
+    if slot.numel() != T or pos.numel() != T:
+        raise ValueError("normattn_prepare: one slot and position per row")
+    _check(load_library().lgs_normattn_prepare(_dev(proj, "proj", F32), ld, q_off, k_off, v_off,
+                                               _dev(cache_k, "cache_k"), _dev(cache_v, "cache_v"),
+                                               _wf32(cache_k, "cache_k"), _dev(slot, "slot", I32),
+                                               _dev(pos, "pos", I32), T, H, G, d, dv, S, float(eps), float(temp_coef),
+                                               int(temp_every), _stream()))
+
+
+def sinkattn(proj: torch.Tensor, q_off: int, cache_k: torch.Tensor, cache_v: torch.Tensor,
+             sink: Optional[torch.Tensor], seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor,
+             max_len: int, *, H: int, G: int, d: int, dv: int, scale: float, chunk: int = 0, cap: float = 0.0,
+             post: float = 1.0, bf16_copy: bool = False, splits: Optional[int] = None) -> torch.Tensor:
+    """Causal softmax attention of every row of a packed batch over its sequence's cached keys and values, grouped
+    key / value heads, with exp(sink[h]) in the normaliser; the prepared queries are the H d columns of ``proj`` at
+    ``q_off``. Returns (T, H dv) fp32 times ``post``, or with ``bf16_copy`` its rounding to bf16."""
+    T, ld = proj.shape
+    B = seq_slot.numel()
+    slots, S = cache_k.shape[:2]
+    if tuple(cache_k.shape) != (slots, S, G, d) or tuple(cache_v.shape) != (slots, S, G, dv):
+        raise ValueError("sinkattn: cache shapes")
+    if seq_start.numel() != B + 1 or q_off + H * d > ld or not 1 <= max_len <= T or \
+            (sink is not None and sink.numel() != H):
+        raise ValueError("sinkattn: step table / query columns / sink")
+    out = torch.empty(T, H * dv, dtype=F32, device=proj.device)
+    out16 = torch.empty(T, H * dv, dtype=torch.bfloat16, device=proj.device) if bf16_copy else None
+    if max_len > 1:
+        splits = 1
+    elif splits is None:
+        span = min(S, chunk) if chunk > 0 else S
+        splits = max(1, min(64, 512 // max(1, B * H), (span + 127) // 128))
+    part = torch.empty(T * H * splits * (2 + dv), dtype=F32, device=proj.device) if splits > 1 else None
+    _check(load_library().lgs_sinkattn(_dev(proj, "proj", F32) + 4 * q_off, ld, _dev(cache_k, "cache_k"),
+                                       _dev(cache_v, "cache_v"), _wf32(cache_k, "cache_k"), _opt(sink, "sink", F32),
+                                       _dev(seq_start, "seq_start", I32), _dev(seq_slot, "seq_slot", I32),
+                                       _dev(seq_pos0, "seq_pos0", I32), out.data_ptr(),
+                                       _opt(out16, "out_bf16", torch.bfloat16), _opt(part, "part", F32), splits, B,
+                                       int(max_len), H, G, d, dv, S, int(chunk), float(scale), float(cap), float(post),
+                                       _stream()))
+    return out16 if bf16_copy else out
+
+
+def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tensor, b_off: int, A_log: torch.Tensor,
+                  dt_bias: torch.Tensor, *, H: int, G: int, d: int, per_channel: bool, q_scale: float,
+                  norm_eps: float = 1e-6):
+    """qkv (T, 2 G d + H dv): q and k become unit vectors per head in place (q also times ``q_scale``). The raw decay
+    inputs are the H d (``per_channel``) or H columns of ``a`` at ``a_off``, the raw betas the H columns of ``b`` at
+    ``b_off``. Returns (dec, beta): exp(-exp(A_log) softplus(a + dt_bias)) (T, H d) or (T, H), sigmoid(b) (T, H)."""
+    T, ld = qkv.shape
+    n = H * d if per_channel else H
+    if a.shape[0] != T or b.shape[0] != T or a_off + n > a.shape[1] or b_off + H > b.shape[1] or \
+            A_log.numel() != H or dt_bias.numel() != n or ld < 2 * G * d:
+        raise ValueError("delta_prepare: shapes")
+    dec = torch.empty(T, n, dtype=F32, device=qkv.device)
+    beta = torch.empty(T, H, dtype=F32, device=qkv.device)
+    _check(load_library().lgs_delta_prepare(_dev(qkv, "qkv", F32), ld, _dev(a, "a", F32) + 4 * a_off, a.shape[1],
+                                            _dev(b, "b", F32) + 4 * b_off, b.shape[1], _dev(A_log, "A_log", F32),
+                                            _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), beta.data_ptr(), T, H, G, d,
+                                            int(per_channel), float(q_scale), float(norm_eps), _stream()))
+    return dec, beta
+
+
+def gated_delta(qkv: torch.Tensor, dec: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, seq_start: torch.Tensor,
+                seq_slot: torch.Tensor, seq_pos0: torch.Tensor, *, H: int, G: int, d: int, dv: int,
+                per_channel: bool, lanes: int = 0) -> torch.Tensor:
+    """The gated delta rule over a packed batch, token by token: S <- diag(dec) S; u = beta (v - S^T k);
+    S <- S + k u^T; o = S^T q. qkv (T, 2 G d + H dv) prepared rows; state (slots, H, d, dv) fp32 is read unless a
+    sequence starts at position 0 and left at the step's last token. Returns o (T, H dv). ``lanes``: lanes that share
+    one state column (4, 8, 16; 0: chosen from the sizes)."""
+    T, ld = qkv.shape
+    B = seq_slot.numel()
+    if ld != 2 * G * d + H * dv or tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or \
+            dec.shape != (T, H * d if per_channel else H) or beta.shape != (T, H):
+        raise ValueError("gated_delta: shapes")
+    out = torch.empty(T, H * dv, dtype=F32, device=qkv.device)
+    _check(load_library().lgs_gated_delta(_dev(qkv, "qkv", F32), ld, _dev(dec, "dec", F32), _dev(beta, "beta", F32),
+                                          _dev(state, "state", F32), _dev(seq_start, "seq_start", I32),
+                                          _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32),
+                                          out.data_ptr(), B, H, G, d, dv, int(per_channel), int(lanes), _stream()))
     return out
