@@ -258,3 +258,105 @@ def test_rigulorn_plain_implementation_is_causal_and_chunked():
     u = torch.arange(6.0, dtype=torch.float64).view(6, 1)
     got = orc.causal_conv(u, torch.tensor([[0.0, 0.0, 1.0]], dtype=torch.float64), torch.zeros(1, dtype=torch.float64))
     assert torch.equal(got, u)
+
+
+# ------------------------------------------------------------------------------------------------ Ravelorn
+def _rav_cfg():
+    return {
+        "architecture": "Ravelorn", "vocab": 23, "width": 16, "norm": {"eps": 1e-5}, "residual_mult": 0.4,
+        "logit_softcap": 7.0, "max_positions": 30,
+        "layers": [
+            {"type": "channel_delta", "mlp": {"kind": "moe", "expert": {"ff": 6}, "router": {"experts": 3, "identity": 2, "top": 2}},
+             "mixer": {"heads": 4, "kv_heads": 2, "dim": 6, "vdim": 5, "conv": 3, "decay_rank": 3, "gate_rank": 4}},
+            {"type": "parallel", "mlp": None,
+             "mixer": {"left": {"heads": 6, "kv_heads": 2, "dim": 4, "vdim": 3, "scale": 0.3, "q_temp": {"coef": 0.5, "every": 4}},
+                       "right": {"heads": 2, "kv_heads": 1, "dim": 8, "vdim": 6, "conv": 2},
+                       "left_scale": 1.5, "right_scale": 0.25}},
+        ]}
+
+
+def test_ravelorn_config_and_tensor_names():
+    from lit_gpt.config import LayeredConfig, model_class
+    from lit_gpt.layered import LayeredGPT
+
+    c = LayeredConfig.from_dict(_rav_cfg())
+    assert model_class(c) is LayeredGPT
+    d = c.design
+    assert (d.block, d.norm, d.positions, d.moe, d.tied_head) == ("post", "layer", "learned", "scores", False)
+    assert (c.residual_mult, c.logit_softcap, c.max_positions) == (0.4, 7.0, 30)
+    a, p = (l.mixer for l in c.layers)
+    assert (a.kind, a.heads, a.kv_heads, a.dim, a.vdim, a.conv) == ("channel_delta", 4, 2, 6, 5, 3)
+    assert (p.left.kind, p.left.heads, p.left.kv_heads, p.left.scale, p.left.q_temp_coef, p.left.q_temp_every) == \
+        ("sink_attention", 6, 2, 0.3, 0.5, 4)
+    assert (p.right.kind, p.right.heads, p.right.kv_heads, p.right.conv, p.left_scale, p.right_scale) == \
+        ("gated_delta", 2, 1, 2, 1.5, 0.25)
+    f = c.layers[0].mlp
+    assert (f.experts, f.identity, f.top, f.ff) == (3, 2, 2, 6) and c.layers[1].mlp is None
+    shapes = LayeredGPT.tensor_shapes(c)
+    assert shapes["pos"] == (30, 16) and shapes["head"] == (23, 16) and shapes["final.norm.b"] == (16,)
+    assert shapes["l0.norm1.b"] == (16,) and shapes["l0.norm2.b"] == (16,) and "l1.norm2" not in shapes
+    assert shapes["l0.mix.q"] == (12, 16) and shapes["l0.mix.v"] == (20, 16) and shapes["l0.mix.k.conv"] == (12, 3)
+    assert shapes["l0.mix.a1"] == (3, 16) and shapes["l0.mix.a2"] == (24, 3) and shapes["l0.mix.dt_bias"] == (24,)
+    assert shapes["l0.mix.g2"] == (20, 4) and shapes["l0.mix.norm"] == (5,) and shapes["l0.mix.b"] == (4, 16)
+    assert shapes["l0.mlp.router"] == (5, 16) and shapes["l0.mlp.correction"] == (5,) and "l0.mlp.e3.up" not in shapes
+    assert shapes["l0.mlp.e2.gate"] == (6, 16) and shapes["l0.mlp.e2.down"] == (16, 6)
+    assert shapes["l1.mix.left.q"] == (24, 16) and shapes["l1.mix.left.k"] == (8, 16) and shapes["l1.mix.left.v"] == (6, 16)
+    assert shapes["l1.mix.left.sink"] == (6,) and shapes["l1.mix.left.o"] == (16, 18)
+    assert shapes["l1.mix.right.a"] == (2, 16) and shapes["l1.mix.right.dt_bias"] == (2,) and shapes["l1.mix.right.g"] == (12, 16)
+    w = LayeredGPT.random_weights(c)
+    assert set(w) == set(shapes) and all(tuple(w[k].shape) == shapes[k] for k in shapes)
+    bare = _rav_cfg()
+    del bare["layers"][1]["mixer"]["left"]["q_temp"]
+    assert LayeredConfig.from_dict(bare).layers[1].mixer.left.q_temp_every == 0
+
+
+@pytest.mark.parametrize("edit", [
+    lambda c: c["layers"][0]["mixer"].update(kv_heads=3),  # heads no multiple of the key heads
+    lambda c: c["layers"][0]["mixer"].update(conv=0),
+    lambda c: c["layers"][0]["mixer"].update(dim=600),
+    lambda c: c["layers"][1]["mixer"]["left"].update(kv_heads=4),
+    lambda c: c["layers"][1]["mixer"]["right"].update(kv_heads=0),
+    lambda c: c["layers"][0]["mlp"]["router"].update(top=6),  # more than experts + identity experts
+    lambda c: c.update(max_positions=0),
+])
+def test_ravelorn_config_rejects_what_does_not_fit(edit):
+    from lit_gpt.config import LayeredConfig
+
+    c = _rav_cfg()
+    edit(c)
+    with pytest.raises(ValueError):
+        LayeredConfig.from_dict(c)
+
+
+def test_ravelorn_plain_implementation():
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+    from oracle import ravelorn as orc
+
+    cfg = _rav_cfg()
+    w = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=3)
+    toks = [3, 7, 1, 0, 22, 5, 9, 9, 4, 13, 2, 8]
+    full = orc.forward(cfg, w, toks)
+    assert torch.allclose(orc.forward(cfg, w, toks[:7]), full[:7], atol=1e-10)  # causal
+    assert float(full.abs().max()) < cfg["logit_softcap"]
+    # a convolution kernel that is 1 in column taps - 1 and 0 elsewhere passes its input to the activation
+    u = torch.linspace(-2, 2, 6, dtype=torch.float64).view(6, 1)
+    assert torch.allclose(orc.causal_conv_silu(u, torch.tensor([[0.0, 0.0, 1.0]], dtype=torch.float64)), orc.silu(u))
+    # the delta rule stores a value under a key and returns it to a query along that key; a second write under the
+    # same key replaces it (beta 1, no decay)
+    k = torch.tensor([[1.0, 0.0], [1.0, 0.0], [0.0, 1.0]], dtype=torch.float64)
+    v = torch.tensor([[2.0, 3.0], [5.0, 7.0], [1.0, 1.0]], dtype=torch.float64)
+    o = orc.delta_rule(k, k, v, torch.ones(3, dtype=torch.float64), torch.ones(3, 2, dtype=torch.float64))
+    assert torch.allclose(o, v)
+    # a sink as large as the only score halves the output; identity experts return the input
+    m = {"heads": 1, "kv_heads": 1, "dim": 2, "vdim": 2, "scale": 1.0}
+    eye = torch.eye(2, dtype=torch.float64)
+    h = torch.tensor([[1.0, 1.0]], dtype=torch.float64)
+    aw = {"q": eye, "k": eye, "v": eye, "o": eye}
+    plain = orc.sink_attention(h, aw, m, 0.0)
+    score = 2.0  # unit-RMS q . k
+    halved = orc.sink_attention(h, dict(aw, sink=torch.tensor([score], dtype=torch.float64)), m, 0.0)
+    assert torch.allclose(plain, h) and torch.allclose(halved, 0.5 * h)
+    rw = {"router": torch.tensor([[0.0, 0.0], [9.0, 9.0]], dtype=torch.float64)}
+    out = orc.moe_ff(h, rw, {"router": {"experts": 0, "identity": 2, "top": 1}})
+    assert torch.allclose(out, torch.softmax(torch.tensor([0.0, 18.0], dtype=torch.float64), 0)[1] * h)
