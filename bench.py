@@ -607,6 +607,120 @@ def hybrid_bench(args) -> None:
         print(json.dumps(line), flush=True)
 
 
+def _layered_timings(model, args, T: int, V: int) -> dict:
+    """Prefill throughput (one prompt step, warm, median of 3) and captured greedy decode steps at context T of a
+    layered model through ``BatchEngine``, for 1 and 8 sequences."""
+    from generate.batch import BatchEngine
+
+    steps = args.steps
+    g = torch.Generator().manual_seed(1234)
+    res = {}
+
+    def timed(fn, reps=3):
+        out = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            out.append(time.perf_counter() - t0)
+        return sorted(out)[len(out) // 2]
+
+    for B in (1, 8):
+        eng = BatchEngine(model, max_seq_length=T + steps + args.warmup + 8, slots=B)
+        prompts = [torch.randint(0, V, (T,), generator=g).tolist() for _ in range(B)]
+        ids = list(range(B))
+        with torch.inference_mode():
+            def prefill():
+                for r in list(eng.live):
+                    eng.step([], end=[r])
+                return eng.step([(i, prompts[i], [T - 1]) for i in ids])
+            prefill()
+            res[f"prefill_tok_s_b{B}"] = round(B * T / timed(prefill))
+            lg = prefill()
+            first = [int(torch.argmax(lg[i])) for i in ids]
+            graph = eng.decode_graph(ids, first)
+            graph.step()
+            for _ in range(args.warmup):
+                graph.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                graph.step()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / steps
+        res[f"decode_tok_s_b{B}"] = round(B / dt, 1)
+        res[f"decode_ms_step_b{B}"] = round(dt * 1e3, 4)
+        del eng, graph
+        model.clear_kv_cache()
+    return res
+
+
+def delta_bench(args) -> None:
+    """``--delta``: prefill and decode throughput of the Ravelorn design (gated-delta-rule layers with per-channel
+    decay alternating with layers that run a sink attention and a per-head-decay delta rule side by side, every
+    layer with score-routed gated experts; random bf16 weights) at sizes that resemble a real model's layers, beside
+    the closest existing model of the framework - the Rigulorn layers (state-space scans and differential attention,
+    dense feed-forwards, here on one residual stream) - at equal width, depth, head count and active feed-forward
+    size. One JSON line per size: one 2048-token prompt (warm, median of 3) and captured greedy decode steps at
+    context 2048, for 1 and 8 sequences. ``hbm_frac``: algorithmic bytes of a one-sequence decode step over 8 TB/s."""
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+
+    dev = torch.device("cuda", 0)
+    T, L, V = args.prompt_len, 4, 32000
+    sizes = {"w2048": (2048, 5632), "w4096": (4096, 11008)}
+    for name, (W, ff) in sizes.items():
+        if args.delta not in ("all", name):
+            continue
+        H = W // 128
+        E, top, ident = 16, 4, 2
+        moe = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": E, "identity": ident, "top": top}}
+        cd = {"type": "channel_delta", "mixer": {"heads": H, "kv_heads": H, "dim": 128, "vdim": 128, "conv": 4,
+                                                 "decay_rank": W // 32, "gate_rank": W // 32}, "mlp": moe}
+        par = {"type": "parallel", "mlp": moe, "mixer": {
+            "left": {"heads": H, "kv_heads": H // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "q_temp": {"coef": 0.1, "every": 512}},
+            "right": {"heads": H // 2, "kv_heads": H // 2, "dim": 128, "vdim": 128, "conv": 4},
+            "left_scale": 1.0, "right_scale": 1.0}}
+        cfg = LayeredConfig.from_dict({"architecture": "Ravelorn", "vocab": V, "width": W, "norm": {"eps": 1e-5},
+                                       "residual_mult": 0.7, "logit_softcap": 30.0, "max_positions": 4096,
+                                       "layers": [cd, par, cd, par]})
+        line = {"bench": "delta", "size": name, "width": W, "ff": ff, "layers": L, "prompt_len": T, "steps": args.steps,
+                "dtype": "bf16", "data": "synthetic"}
+        model = LayeredGPT(cfg, LayeredGPT.random_weights(cfg, seed=1), device=dev, dtype=torch.bfloat16)
+        res = _layered_timings(model, args, T, V)
+        # algorithmic traffic of a decode step (B = 1): every dense matrix once in bf16, the chosen experts, the cached
+        # keys and values of the attention halves (bf16), the recurrent states (fp32, read and written)
+        dense = 0
+        for blk in model.blocks:
+            dense += blk.sub1.w_in.numel() + blk.sub2.w_in.numel()
+            mixers = [blk.mixer.left, blk.mixer.right] if hasattr(blk.mixer, "left") else [blk.mixer]
+            dense += sum(m.w_o.numel() + sum(getattr(m, n).numel() for n in ("w_a2", "w_g2") if hasattr(m, n)) for m in mixers)
+        experts = L * top * 3 * W * (ff // top)
+        kv = 2 * T * (H // 4) * (128 + 128) * 2
+        state = 2 * (2 * H + 2 * (H // 2)) * 128 * 128 * 4
+        res["hbm_frac_decode_b1"] = round((2 * (dense + experts + V * W) + kv + state) / (res["decode_ms_step_b1"] * 1e-3)
+                                          / (HBM_PEAK_GBS * 1e9), 3)
+        line["ravelorn"] = res
+        del model
+        torch.cuda.empty_cache()
+        att = {"heads": H, "kv_heads": H // 4, "dim": 64, "vdim": 128, "diff": 0.5, "softcap": 30.0, "scale": 0.125,
+               "rot": {"dims": 64, "base": 1e4}}
+        ssm = {"type": "mamba2", "mixer": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8,
+                                           "conv": 4}}
+        mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+        rcfg = LayeredConfig.from_dict({
+            "architecture": "Rigulorn", "vocab": V, "width": W, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "layers": [dict(ssm, mlp=mlp), {"type": "attention", "mixer": att, "mlp": mlp}, dict(ssm, mlp=mlp),
+                       {"type": "attention", "mixer": att, "mlp": mlp}]})
+        model = LayeredGPT(rcfg, LayeredGPT.random_weights(rcfg, seed=1), device=dev, dtype=torch.bfloat16)
+        line["rigulorn_layers"] = _layered_timings(model, args, T, V)
+        del model
+        torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -616,6 +730,9 @@ def main():
     ap.add_argument("--hybrid", nargs="?", const="all", default=None, choices=("all", "w2048", "w4096"),
                     help="instead of the headline run: the Rigulorn design (state-space and differential-attention "
                          "layers over several residual streams) beside a Llama-family stack of equal size")
+    ap.add_argument("--delta", nargs="?", const="all", default=None, choices=("all", "w2048", "w4096"),
+                    help="instead of the headline run: the Ravelorn design (gated delta rule, sink attention, routed "
+                         "experts) beside the Rigulorn layers at equal size")
     # defaults: the eager capture step (p = 2048) + 14 warm-up + 240 timed steps = the 255 decode steps of
     # SURVEY §8d (p = 2048 ... 2302)
     ap.add_argument("--steps", type=int, default=240)
@@ -639,6 +756,8 @@ def main():
         return layered_bench(args)
     if args.hybrid:
         return hybrid_bench(args)
+    if args.delta:
+        return delta_bench(args)
     traffic = {k: (None, "skipped") for k in ("gemv", "attention")}
     under_profiler = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
     headline = args.model == MODEL and args.quantize == "int4-g128"

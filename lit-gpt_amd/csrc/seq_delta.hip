@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
   constexpr int CW = 256 / LPC;          // columns per workgroup
   constexpr int ROW = 3 * DP + CW + 4;   // staged floats per token: q | k | g | v | beta (rows stay 16-byte aligned)
   constexpr int kDeltaTB = DP > 256 ? 8 : 16;  // tokens staged at a time
-  constexpr int PRE = (kDeltaTB * ROW + 255) / 256;
+  constexpr int EPT = (ROW + 255) / 256;       // staged entries per thread and token
   __shared__ __attribute__((aligned(16))) float st[kDeltaTB * ROW];
   __shared__ float os[kDeltaTB][CW];
   const int tid = threadIdx.x;
@@ -111,40 +111,48 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
       const int row = 4 * (r + LPC * j) + e;
       S[j][e] = (!fresh && live && row < d) ? sp[(size_t)row * dv + col] : 0.0f;
     }
-  const size_t qo = (size_t)g * d, ko = (size_t)(p.G + g) * d, vo = (size_t)2 * p.G * d + (size_t)hd * dv + blockIdx.x * CW;
-
-  // staged item idx of the batch that starts at token t0: token idx / ROW, entry idx % ROW
-  auto fetch = [&](int t0, int idx) -> float {
-    const int t = idx / ROW, e = idx % ROW;
-    if (idx >= kDeltaTB * ROW || t0 + t >= n) return 0.0f;
-    const size_t rw = (size_t)(r0 + t0 + t);
-    if (e < DP) return e < d ? p.qkv[rw * p.ld + qo + e] : 0.0f;
-    if (e < 2 * DP) return e - DP < d ? p.qkv[rw * p.ld + ko + (e - DP)] : 0.0f;
-    if (e < 3 * DP) {
-      const int c = e - 2 * DP;
-      return c < d ? p.dec[(rw * H + hd) * dc + (dc == 1 ? 0 : c)] : 1.0f;
-    }
-    if (e < 3 * DP + CW) {
-      const int c = e - 3 * DP;
-      return blockIdx.x * CW + c < dv ? p.qkv[rw * p.ld + vo + c] : 0.0f;
-    }
-    return p.beta[rw * H + hd];
-  };
-  float pre[PRE];
+  // Entry e = tid + 256 i of a token's staged row comes from one place whatever the token: a pointer to it at the
+  // sequence's first row, the distance to the next token's, and the value of an entry that has no source (padding).
+  const float* src[EPT];
+  long step[EPT];
+  float pad[EPT];
 #pragma unroll
-  for (int i = 0; i < PRE; ++i) pre[i] = fetch(0, tid + 256 * i);
+  for (int i = 0; i < EPT; ++i) {
+    const int e = tid + 256 * i;
+    src[i] = nullptr, step[i] = 0, pad[i] = 0.0f;
+    if (e < 2 * DP) {  // q, then k
+      const int c = e < DP ? e : e - DP;
+      if (c < d) src[i] = p.qkv + (size_t)r0 * p.ld + (size_t)((e < DP ? g : p.G + g)) * d + c, step[i] = p.ld;
+    } else if (e < 3 * DP) {
+      const int c = e - 2 * DP;
+      pad[i] = 1.0f;
+      if (c < d) src[i] = p.dec + ((size_t)r0 * H + hd) * dc + (dc == 1 ? 0 : c), step[i] = (long)H * dc;
+    } else if (e < 3 * DP + CW) {
+      const int c = blockIdx.x * CW + (e - 3 * DP);
+      if (c < dv) src[i] = p.qkv + (size_t)r0 * p.ld + (size_t)2 * p.G * d + (size_t)hd * dv + c, step[i] = p.ld;
+    } else if (e == 3 * DP + CW) {
+      src[i] = p.beta + (size_t)r0 * H + hd, step[i] = H;
+    }
+  }
+  float pre[kDeltaTB][EPT];
+  auto prefetch = [&](int t0) {
+#pragma unroll
+    for (int t = 0; t < kDeltaTB; ++t)
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) pre[t][i] = (src[i] && t0 + t < n) ? src[i][(size_t)(t0 + t) * step[i]] : pad[i];
+  };
+  prefetch(0);
 
   for (int t0 = 0; t0 < n; t0 += kDeltaTB) {
     const int nb = min(kDeltaTB, n - t0);
     __syncthreads();  // the previous batch's reads of st and os are done
 #pragma unroll
-    for (int i = 0; i < PRE; ++i)
-      if (tid + 256 * i < kDeltaTB * ROW) st[tid + 256 * i] = pre[i];
-    __syncthreads();
-    if (t0 + kDeltaTB < n) {
+    for (int t = 0; t < kDeltaTB; ++t)
 #pragma unroll
-      for (int i = 0; i < PRE; ++i) pre[i] = fetch(t0 + kDeltaTB, tid + 256 * i);
-    }
+      for (int i = 0; i < EPT; ++i)
+        if (tid + 256 * i < ROW) st[t * ROW + tid + 256 * i] = pre[t][i];
+    __syncthreads();
+    if (t0 + kDeltaTB < n) prefetch(t0 + kDeltaTB);
     for (int t = 0; t < nb; ++t) {
       const float* row = st + t * ROW;
       float ks = 0.0f;

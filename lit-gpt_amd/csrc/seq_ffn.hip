@@ -16,6 +16,50 @@
 
 namespace lgs {
 
+// eight consecutive weights starting at element i (i % 8 == 0, 16-byte aligned rows): one 16-byte load for bf16
+template <bool WF32>
+__device__ __forceinline__ void wload8(const void* w, size_t i, float* o) {
+  if (WF32) {
+    const float4 a = *(const float4*)((const float*)w + i), b = *(const float4*)((const float*)w + i + 4);
+    o[0] = a.x, o[1] = a.y, o[2] = a.z, o[3] = a.w, o[4] = b.x, o[5] = b.y, o[6] = b.z, o[7] = b.w;
+  } else {
+    const uint4 a = *(const uint4*)((const uint16_t*)w + i);
+    o[0] = bflo(a.x), o[1] = bfhi(a.x), o[2] = bflo(a.y), o[3] = bfhi(a.y);
+    o[4] = bflo(a.z), o[5] = bfhi(a.z), o[6] = bflo(a.w), o[7] = bfhi(a.w);
+  }
+}
+// the dot products of one activation row (fp32, rounded as the weights' precision asks) with two weight rows of n
+// elements; `vec` (n % 8 == 0 and 16-byte aligned rows) takes 16-byte loads
+template <bool WF32>
+__device__ __forceinline__ void dot2(const float* __restrict__ x, const void* __restrict__ w, size_t r0, size_t r1, int n,
+                                     bool vec, int lane, float& a0, float& a1) {
+  a0 = a1 = 0.0f;
+  if (vec) {
+#pragma unroll 2
+    for (int k = lane * 8; k < n; k += 512) {
+      float u[8], v[8];
+      wload8<WF32>(w, r0 + k, u);
+      wload8<WF32>(w, r1 + k, v);
+      const float4 xa = *(const float4*)(x + k), xb = *(const float4*)(x + k + 4);
+      const float xs[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xe = aop<WF32>(xs[e]);
+        a0 = fmaf(xe, u[e], a0);
+        a1 = fmaf(xe, v[e], a1);
+      }
+    }
+  } else {
+    for (int k = lane; k < n; k += 64) {
+      const float xe = aop<WF32>(x[k]);
+      a0 = fmaf(xe, wload<WF32>(w, r0 + k), a0);
+      a1 = fmaf(xe, wload<WF32>(w, r1 + k), a1);
+    }
+  }
+  a0 = wave_sum(a0);
+  a1 = wave_sum(a1);
+}
+
 __global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ a, const float* __restrict__ b, long ld,
                                                   float* __restrict__ out, uint16_t* __restrict__ out16, int n, int act) {
   const size_t t = blockIdx.x;
@@ -161,14 +205,8 @@ __global__ void __launch_bounds__(256) moe_up_kernel(const float* __restrict__ h
   const float* hr = h + (size_t)(pair / top) * ldh;
   const size_t rows = GATED ? 2 * (size_t)F : (size_t)F;
   const size_t w0 = ((size_t)e * rows + f0) * K, w1 = ((size_t)e * rows + (GATED ? F + f0 : min(f0 + 1, F - 1))) * K;
-  float a0 = 0.0f, a1 = 0.0f;
-  for (int k = lane; k < K; k += 64) {
-    const float x = aop<WF32>(hr[k]);
-    a0 = fmaf(x, wload<WF32>(up, w0 + k), a0);
-    a1 = fmaf(x, wload<WF32>(up, w1 + k), a1);
-  }
-  a0 = wave_sum(a0);
-  a1 = wave_sum(a1);
+  float a0, a1;
+  dot2<WF32>(hr, up, w0, w1, K, (K & 7) == 0 && (ldh & 3) == 0 && ((uintptr_t)h & 15) == 0, lane, a0, a1);
   if (lane == 0) {
     if (GATED) {
       actbuf[(size_t)pair * F + f0] = act_f(act, a0) * a1;
@@ -201,15 +239,11 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const float* __restrict__
     }
     const float* ar = actbuf + ((size_t)t * top + k) * F;
     const size_t w0 = ((size_t)e * N + n0) * F, w1 = ((size_t)e * N + min(n0 + 1, N - 1)) * F;
-    float a0 = 0.0f, a1 = 0.0f;
-    for (int f = lane; f < F; f += 64) {
-      const float a = aop<WF32>(ar[f]);
-      a0 = fmaf(a, wload<WF32>(down, w0 + f), a0);
-      a1 = fmaf(a, wload<WF32>(down, w1 + f), a1);
-    }
+    float a0, a1;
+    dot2<WF32>(ar, down, w0, w1, F, (F & 7) == 0, lane, a0, a1);
     const float w = wts[(size_t)t * top + k];
-    y0 = fmaf(w, wave_sum(a0), y0);
-    y1 = fmaf(w, wave_sum(a1), y1);
+    y0 = fmaf(w, a0, y0);
+    y1 = fmaf(w, a1, y1);
   }
   if (lane == 0) {
     x[(size_t)t * ldx + n0] = accumulate ? x[(size_t)t * ldx + n0] + y0 : y0;
