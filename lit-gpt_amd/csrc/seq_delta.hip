@@ -88,7 +88,7 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
   constexpr int DP = 4 * NR4 * LPC;      // rows, padded
   constexpr int CW = 256 / LPC;          // columns per workgroup
   constexpr int ROW = 3 * DP + CW + 4;   // staged floats per token: q | k | g | v | beta (rows stay 16-byte aligned)
-  constexpr int kDeltaTB = DP > 256 ? 8 : 16;  // tokens staged at a time
+  constexpr int kDeltaTB = DP > 256 ? 8 : (DP > 128 ? 16 : 32);  // tokens staged at a time
   constexpr int EPT = (ROW + 255) / 256;       // staged entries per thread and token
   __shared__ __attribute__((aligned(16))) float st[kDeltaTB * ROW];
   __shared__ float os[kDeltaTB][CW];
@@ -153,10 +153,13 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
         if (tid + 256 * i < ROW) st[t * ROW + tid + 256 * i] = pre[t][i];
     __syncthreads();
     if (t0 + kDeltaTB < n) prefetch(t0 + kDeltaTB);
+    // (four partial sums per dot product keep the dependent chains short; two tokens per trip let the read-out of
+    // one token overlap the decay and key product of the next)
+#pragma unroll 2
     for (int t = 0; t < nb; ++t) {
       const float* row = st + t * ROW;
-      float ks = 0.0f;
       float4 k4[NR4];
+      float ka = 0.0f, kb = 0.0f, kc = 0.0f, kd = 0.0f;
 #pragma unroll
       for (int j = 0; j < NR4; ++j) {
         const int at = 4 * (r + LPC * j);
@@ -166,14 +169,14 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
         S[j][1] *= g4.y;
         S[j][2] *= g4.z;
         S[j][3] *= g4.w;
-        ks = fmaf(S[j][0], k4[j].x, ks);
-        ks = fmaf(S[j][1], k4[j].y, ks);
-        ks = fmaf(S[j][2], k4[j].z, ks);
-        ks = fmaf(S[j][3], k4[j].w, ks);
+        ka = fmaf(S[j][0], k4[j].x, ka);
+        kb = fmaf(S[j][1], k4[j].y, kb);
+        kc = fmaf(S[j][2], k4[j].z, kc);
+        kd = fmaf(S[j][3], k4[j].w, kd);
       }
-      ks = lanes_sum<LPC>(ks);
+      const float ks = lanes_sum<LPC>((ka + kb) + (kc + kd));
       const float u = row[3 * DP + CW] * (row[3 * DP + cw] - ks);
-      float o = 0.0f;
+      float oa = 0.0f, ob = 0.0f, oc = 0.0f, od = 0.0f;
 #pragma unroll
       for (int j = 0; j < NR4; ++j) {
         const float4 q4 = *(const float4*)(row + 4 * (r + LPC * j));
@@ -181,12 +184,12 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
         S[j][1] = fmaf(k4[j].y, u, S[j][1]);
         S[j][2] = fmaf(k4[j].z, u, S[j][2]);
         S[j][3] = fmaf(k4[j].w, u, S[j][3]);
-        o = fmaf(S[j][0], q4.x, o);
-        o = fmaf(S[j][1], q4.y, o);
-        o = fmaf(S[j][2], q4.z, o);
-        o = fmaf(S[j][3], q4.w, o);
+        oa = fmaf(S[j][0], q4.x, oa);
+        ob = fmaf(S[j][1], q4.y, ob);
+        oc = fmaf(S[j][2], q4.z, oc);
+        od = fmaf(S[j][3], q4.w, od);
       }
-      o = lanes_sum<LPC>(o);
+      const float o = lanes_sum<LPC>((oa + ob) + (oc + od));
       if (r == 0) os[t][cw] = o;
     }
     __syncthreads();
