@@ -180,16 +180,17 @@ int lgs_sinkattn(const float* q, long ld, const void* cache_k, const void* cache
 /* Per token, on rows qkv [T][ld] = q [G][d] | k [G][d] | v [H][dv] (after their convolution): q and k become unit
  * vectors per head, x / sqrt(sum(x^2) + norm_eps), q also times q_scale, in place; beta[t][h] = sigmoid(b[t ldb + h]);
  * dec = exp(-exp(A_log[h]) softplus(a + dt_bias)) with a, dt_bias and dec per head and key channel ([H][d],
- * per_channel) or per head ([H]). */
+ * per_channel) or per head ([H]); kq[t][g] = k . q of the prepared vectors of key head g. */
 int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb, const float* A_log,
-                      const float* dt_bias, float* dec, float* beta, int T, int H, int G, int d, int per_channel,
-                      float q_scale, float norm_eps, lgs_stream_t stream);
-/* Per sequence and head, token by token: S <- diag(dec) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.
+                      const float* dt_bias, float* dec, float* beta, float* kq, int T, int H, int G, int d,
+                      int per_channel, float q_scale, float norm_eps, lgs_stream_t stream);
+/* Per sequence and head, token by token: S <- diag(dec) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q
+ * (evaluated as S'^T q + u kq on the decayed state S', kq [T][G] = k . q from lgs_delta_prepare).
  * Head h reads q / k head h / (H / G). state [slots][H][d][dv] fp32 is read unless the sequence starts at position 0
  * and written back. d <= 512. lanes: lanes that share a state column (4, 8 or 16; 0: chosen from the sizes). */
-int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, float* state, const int* seq_start,
-                    const int* seq_slot, const int* seq_pos0, float* out, int B, int H, int G, int d, int dv,
-                    int per_channel, int lanes, lgs_stream_t stream);
+int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, const float* kq, float* state,
+                    const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, int B, int H, int G, int d,
+                    int dv, int per_channel, int lanes, lgs_stream_t stream);
 
 /* ---- selective state-space mixer ---- */
 /* out[t][c] = silu(bias[c] + sum_j w[c][j] u[t - (taps - 1 - j)][c]) per sequence of a packed batch; inputs before

@@ -5,10 +5,11 @@
 // groups of value heads (head h reads q / k head h / (H / G)). Everything that enters the recurrence is fp32.
 //
 //   lgs_delta_prepare   per token: q and k (after their convolution) become unit vectors per head, q times q_scale;
-//                       beta = sigmoid(raw); g = exp(-exp(A_log) softplus(raw + dt_bias))
+//                       beta = sigmoid(raw); g = exp(-exp(A_log) softplus(raw + dt_bias)); k . q per key head
 //   lgs_gated_delta     the recurrence, token by token for every step kind. The columns of S never mix, so a column
 //                       is owned by LPC adjacent lanes that hold d / LPC of its rows in registers; the two dot
-//                       products over the rows are summed inside those lanes with DPP adds (no LDS, no barrier);
+//                       products over the rows (both against the decayed state: o = S'^T q + u (k . q)) are summed
+//                       inside those lanes with DPP adds (no LDS, no barrier);
 //                       q, k, g, v, beta of 16 tokens at a time are staged in LDS, the next 16 prefetched in registers
 //                       (8 at a time for key dims above 256)
 #include "seq_common.h"
@@ -27,6 +28,7 @@ struct DeltaPrepArgs {
   const float *A_log, *dt_bias;  // [H]; [H][d] or [H]
   float* dec;                    // [T][H][d] or [T][H]
   float* beta;                   // [T][H]
+  float* kq;                     // [T][G]: k . q of the prepared vectors
   int H, G, d, per_channel;
   float q_scale, norm_eps;
 };
@@ -52,6 +54,14 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
     p.dec[t * n + i] = expf(-rate * softplus_d(p.a[t * p.lda + i] + p.dt_bias[i]));
   }
   for (int h = threadIdx.x; h < p.H; h += 256) p.beta[t * p.H + h] = sigmoid_f(p.b[t * p.ldb + h]);
+  __syncthreads();  // the unit vectors of all heads are written
+  for (int g = wave; g < p.G; g += 4) {
+    const float *q = row + (size_t)g * d, *k = row + (size_t)(p.G + g) * d;
+    float s = 0.0f;
+    for (int i = lane; i < d; i += 64) s = fmaf(q[i], k[i], s);
+    s = wave_sum(s);
+    if (lane == 0) p.kq[t * p.G + g] = s;
+  }
 }
 
 struct DeltaArgs {
@@ -59,10 +69,12 @@ struct DeltaArgs {
   long ld;
   const float* dec;   // [T][H][dc], dc = d or 1
   const float* beta;  // [T][H]
+  const float* kq;    // [T][G]
   float* state;       // [slots][H][d][dv]
   const int *seq_start, *seq_slot, *seq_pos0;
   float* out;  // [T][H * dv]
   int H, G, d, dv, per_channel;
+  int ncb, items;  // column blocks per head; work items = B * H * ncb
 };
 
 template <int CTRL>
@@ -70,18 +82,24 @@ __device__ __forceinline__ float dpp_f(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
 // sum over LPC adjacent lanes (aligned, inside a row of 16 lanes); every lane of the group gets the sum. The order
-// of the additions is fixed: neighbours, pairs, then the mirrored halves.
+// of the additions is fixed: neighbours, pairs, then the mirrored halves. Two values at once: their steps interleave.
 template <int LPC>
-__device__ __forceinline__ float lanes_sum(float v) {
-  v += dpp_f<0xB1>(v);                  // quad_perm [1, 0, 3, 2]
-  v += dpp_f<0x4E>(v);                  // quad_perm [2, 3, 0, 1]
-  if (LPC >= 8) v += dpp_f<0x141>(v);   // row_half_mirror: lane i of 8 with lane 7 - i
-  if (LPC >= 16) v += dpp_f<0x140>(v);  // row_mirror: lane i of 16 with lane 15 - i
-  return v;
+__device__ __forceinline__ void lanes_sum2(float& a, float& b) {
+  float x = dpp_f<0xB1>(a), y = dpp_f<0xB1>(b);
+  a += x, b += y;
+  x = dpp_f<0x4E>(a), y = dpp_f<0x4E>(b);
+  a += x, b += y;
+  if (LPC >= 8) {
+    x = dpp_f<0x141>(a), y = dpp_f<0x141>(b);
+    a += x, b += y;
+  }
+  if (LPC >= 16) {
+    x = dpp_f<0x140>(a), y = dpp_f<0x140>(b);
+    a += x, b += y;
+  }
 }
 
-
-// grid (ceil(dv / CW), H, B), CW = 256 / LPC columns per workgroup. Lane l of a wave: r = l % LPC, column
+// grid (B * H * ceil(dv / CW) rounded up to 8), CW = 256 / LPC columns per workgroup. Lane l of a wave: r = l % LPC, column
 // l / LPC of the wave's 64 / LPC; the lane holds the rows 4 (r + LPC j) + e, j < NR4, e < 4, of its column.
 template <int NR4, int LPC>
 __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
@@ -94,8 +112,13 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
   __shared__ float os[kDeltaTB][CW];
   const int tid = threadIdx.x;
   const int r = tid % LPC, cw = tid / LPC;  // cw: column inside the workgroup
-  const int hd = blockIdx.y, b = blockIdx.z;
-  const int col = blockIdx.x * CW + cw;
+  // Workgroups are dealt to the 8 XCDs in turn. The column blocks of one (sequence, head) read the same q, k and
+  // decays, so consecutive work items go to ONE XCD (and its L2): item = xcd * per_xcd + turn.
+  const int per_xcd = (p.items + 7) / 8;
+  const int item = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (item >= p.items) return;
+  const int cblk = item % p.ncb, hd = (item / p.ncb) % p.H, b = item / (p.ncb * p.H);
+  const int col = cblk * CW + cw;
   const int d = p.d, dv = p.dv, H = p.H;
   const bool live = col < dv;
   const int g = hd / (H / p.G);
@@ -113,9 +136,11 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
     }
   // Entry e = tid + 256 i of a token's staged row comes from one place whatever the token: a pointer to it at the
   // sequence's first row, the distance to the next token's, and the value of an entry that has no source (padding).
+  // (an entry without a source loads a valid address all the same, so that the loads carry no branches)
   const float* src[EPT];
   long step[EPT];
   float pad[EPT];
+  bool has[EPT];
 #pragma unroll
   for (int i = 0; i < EPT; ++i) {
     const int e = tid + 256 * i;
@@ -128,18 +153,25 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
       pad[i] = 1.0f;
       if (c < d) src[i] = p.dec + ((size_t)r0 * H + hd) * dc + (dc == 1 ? 0 : c), step[i] = (long)H * dc;
     } else if (e < 3 * DP + CW) {
-      const int c = blockIdx.x * CW + (e - 3 * DP);
+      const int c = cblk * CW + (e - 3 * DP);
       if (c < dv) src[i] = p.qkv + (size_t)r0 * p.ld + (size_t)2 * p.G * d + (size_t)hd * dv + c, step[i] = p.ld;
     } else if (e == 3 * DP + CW) {
       src[i] = p.beta + (size_t)r0 * H + hd, step[i] = H;
+    } else if (e == 3 * DP + CW + 1) {
+      src[i] = p.kq + (size_t)r0 * p.G + g, step[i] = p.G;
     }
+    has[i] = src[i] != nullptr;
+    if (!has[i]) src[i] = p.beta + (size_t)r0 * H + hd;
   }
   float pre[kDeltaTB][EPT];
   auto prefetch = [&](int t0) {
 #pragma unroll
     for (int t = 0; t < kDeltaTB; ++t)
 #pragma unroll
-      for (int i = 0; i < EPT; ++i) pre[t][i] = (src[i] && t0 + t < n) ? src[i][(size_t)(t0 + t) * step[i]] : pad[i];
+      for (int i = 0; i < EPT; ++i) {
+        const float v = src[i][(size_t)min(t0 + t, n - 1) * step[i]];
+        pre[t][i] = has[i] ? v : pad[i];
+      }
   };
   prefetch(0);
 
@@ -153,18 +185,20 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
         if (tid + 256 * i < ROW) st[t * ROW + tid + 256 * i] = pre[t][i];
     __syncthreads();
     if (t0 + kDeltaTB < n) prefetch(t0 + kDeltaTB);
-    // (four partial sums per dot product keep the dependent chains short; two tokens per trip let the read-out of
-    // one token overlap the decay and key product of the next)
+    // With S' = diag(g) S the output is o = S'^T q + u (k . q): both products with S' run side by side and share one
+    // round of lane sums, and the write S' + k u^T leaves the output's dependent chain. Four partial sums per product
+    // keep the chains short; two tokens per trip let one token's tail overlap the next one's decay.
 #pragma unroll 2
     for (int t = 0; t < nb; ++t) {
       const float* row = st + t * ROW;
       float4 k4[NR4];
-      float ka = 0.0f, kb = 0.0f, kc = 0.0f, kd = 0.0f;
+      float ka = 0.0f, kb = 0.0f, kc = 0.0f, kd = 0.0f, oa = 0.0f, ob = 0.0f, oc = 0.0f, od = 0.0f;
 #pragma unroll
       for (int j = 0; j < NR4; ++j) {
         const int at = 4 * (r + LPC * j);
         k4[j] = *(const float4*)(row + DP + at);
         const float4 g4 = *(const float4*)(row + 2 * DP + at);
+        const float4 q4 = *(const float4*)(row + at);
         S[j][0] *= g4.x;
         S[j][1] *= g4.y;
         S[j][2] *= g4.z;
@@ -173,30 +207,28 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
         kb = fmaf(S[j][1], k4[j].y, kb);
         kc = fmaf(S[j][2], k4[j].z, kc);
         kd = fmaf(S[j][3], k4[j].w, kd);
-      }
-      const float ks = lanes_sum<LPC>((ka + kb) + (kc + kd));
-      const float u = row[3 * DP + CW] * (row[3 * DP + cw] - ks);
-      float oa = 0.0f, ob = 0.0f, oc = 0.0f, od = 0.0f;
-#pragma unroll
-      for (int j = 0; j < NR4; ++j) {
-        const float4 q4 = *(const float4*)(row + 4 * (r + LPC * j));
-        S[j][0] = fmaf(k4[j].x, u, S[j][0]);
-        S[j][1] = fmaf(k4[j].y, u, S[j][1]);
-        S[j][2] = fmaf(k4[j].z, u, S[j][2]);
-        S[j][3] = fmaf(k4[j].w, u, S[j][3]);
         oa = fmaf(S[j][0], q4.x, oa);
         ob = fmaf(S[j][1], q4.y, ob);
         oc = fmaf(S[j][2], q4.z, oc);
         od = fmaf(S[j][3], q4.w, od);
       }
-      const float o = lanes_sum<LPC>((oa + ob) + (oc + od));
-      if (r == 0) os[t][cw] = o;
+      float ks = (ka + kb) + (kc + kd), qs = (oa + ob) + (oc + od);
+      lanes_sum2<LPC>(ks, qs);
+      const float u = row[3 * DP + CW] * (row[3 * DP + cw] - ks);
+      if (r == 0) os[t][cw] = fmaf(u, row[3 * DP + CW + 1], qs);
+#pragma unroll
+      for (int j = 0; j < NR4; ++j) {
+        S[j][0] = fmaf(k4[j].x, u, S[j][0]);
+        S[j][1] = fmaf(k4[j].y, u, S[j][1]);
+        S[j][2] = fmaf(k4[j].z, u, S[j][2]);
+        S[j][3] = fmaf(k4[j].w, u, S[j][3]);
+      }
     }
     __syncthreads();
     for (int i = tid; i < nb * CW; i += 256) {
       const int t = i / CW, c = i % CW;
-      if (blockIdx.x * CW + c < dv)
-        p.out[(size_t)(r0 + t0 + t) * H * dv + (size_t)hd * dv + blockIdx.x * CW + c] = os[t][c];
+      if (cblk * CW + c < dv)
+        p.out[(size_t)(r0 + t0 + t) * H * dv + (size_t)hd * dv + cblk * CW + c] = os[t][c];
     }
   }
   if (live) {
@@ -211,8 +243,10 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
 }
 
 template <int LPC>
-static bool gated_delta_launch(const DeltaArgs& p, int B, hipStream_t stream) {
-  const dim3 grid((p.dv + 256 / LPC - 1) / (256 / LPC), p.H, B);
+static bool gated_delta_launch(DeltaArgs p, int B, hipStream_t stream) {
+  p.ncb = (p.dv + 256 / LPC - 1) / (256 / LPC);
+  p.items = B * p.H * p.ncb;
+  const dim3 grid((p.items + 7) / 8 * 8);
   const int nr4 = (p.d + 4 * LPC - 1) / (4 * LPC);
   if (nr4 <= 1) gated_delta_kernel<1, LPC><<<grid, 256, 0, stream>>>(p);
   else if (nr4 <= 2) gated_delta_kernel<2, LPC><<<grid, 256, 0, stream>>>(p);
@@ -225,23 +259,28 @@ static bool gated_delta_launch(const DeltaArgs& p, int B, hipStream_t stream) {
 }  // namespace lgs
 
 extern "C" int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb,
-                                 const float* A_log, const float* dt_bias, float* dec, float* beta, int T, int H, int G,
-                                 int d, int per_channel, float q_scale, float norm_eps, hipStream_t stream) {
-  LGA_CHECK_ARG(qkv && a && b && A_log && dt_bias && dec && beta && T > 0, "lgs_delta_prepare: bad arguments");
+                                 const float* A_log, const float* dt_bias, float* dec, float* beta, float* kq, int T,
+                                 int H, int G, int d, int per_channel, float q_scale, float norm_eps,
+                                 hipStream_t stream) {
+  LGA_CHECK_ARG(qkv && a && b && A_log && dt_bias && dec && beta && kq && T > 0, "lgs_delta_prepare: bad arguments");
   LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && ld >= 2L * G * d, "lgs_delta_prepare: bad sizes");
-  lgs::DeltaPrepArgs p{qkv, ld, a, lda, b, ldb, A_log, dt_bias, dec, beta, H, G, d, per_channel ? 1 : 0, q_scale, norm_eps};
+  lgs::DeltaPrepArgs p{qkv, ld, a, lda, b, ldb, A_log, dt_bias, dec, beta, kq, H, G, d, per_channel ? 1 : 0, q_scale,
+                       norm_eps};
   lgs::delta_prepare_kernel<<<T, 256, 0, stream>>>(p);
   LGA_LAUNCH_RETURN();
 }
 
-extern "C" int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, float* state,
-                               const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, int B, int H,
-                               int G, int d, int dv, int per_channel, int lanes, hipStream_t stream) {
-  LGA_CHECK_ARG(qkv && dec && beta && state && seq_start && seq_slot && seq_pos0 && out, "lgs_gated_delta: null pointer");
-  LGA_CHECK_ARG(B > 0 && B <= 65535 && H > 0 && H <= 65535 && G > 0 && H % G == 0 && d > 0 && d <= 512 && dv > 0,
+extern "C" int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, const float* kq,
+                               float* state, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
+                               int B, int H, int G, int d, int dv, int per_channel, int lanes, hipStream_t stream) {
+  LGA_CHECK_ARG(qkv && dec && beta && kq && state && seq_start && seq_slot && seq_pos0 && out,
+                "lgs_gated_delta: null pointer");
+  LGA_CHECK_ARG(B > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && d <= 512 && dv > 0,
                 "lgs_gated_delta: bad sizes (key dim <= 512)");
   LGA_CHECK_ARG(ld >= 2L * G * d + (long)H * dv, "lgs_gated_delta: q | k | v outside the row");
-  lgs::DeltaArgs p{qkv, ld, dec, beta, state, seq_start, seq_slot, seq_pos0, out, H, G, d, dv, per_channel ? 1 : 0};
+  LGA_CHECK_ARG((long)B * H * ((dv + 15) / 16) < (1L << 30), "lgs_gated_delta: too many columns");
+  lgs::DeltaArgs p{qkv, ld, dec, beta, kq, state, seq_start, seq_slot, seq_pos0, out, H, G, d, dv, per_channel ? 1 : 0,
+                   0, 0};
   // lanes per column: more lanes shorten a token's dependent chain and multiply the waves; by default as many as
   // keep the launch within about two waves per SIMD, and at least enough for 32 rows per lane
   int lpc = lanes;

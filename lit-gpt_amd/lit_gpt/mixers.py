@@ -339,9 +339,10 @@ class GatedDelta(InputReader):
             a_off, g_off, act = 0, 0, seq_ops.ACT_SIGMOID
         else:
             a, a_off, gate, g_off, act = proj, self.off["a"], proj, self.off["g"], seq_ops.ACT_SILU
-        dec, beta = seq_ops.delta_prepare(qkv, a, a_off, proj, self.off["b"], self.A_log, self.dt_bias, H=H, G=G, d=d,
-                                          per_channel=self.per_channel, q_scale=float(d) ** -0.5)
-        o = seq_ops.gated_delta(qkv, dec, beta, cache.s, *tables, H=H, G=G, d=d, dv=dv, per_channel=self.per_channel)
+        dec, beta, kq = seq_ops.delta_prepare(qkv, a, a_off, proj, self.off["b"], self.A_log, self.dt_bias, H=H, G=G, d=d,
+                                              per_channel=self.per_channel, q_scale=float(d) ** -0.5)
+        o = seq_ops.gated_delta(qkv, dec, beta, kq, cache.s, *tables, H=H, G=G, d=d, dv=dv,
+                                per_channel=self.per_channel)
         o = seq_ops.head_gate(o, gate, g_off, H=H, dv=dv, unit_norm=True, eps=self.eps, act=act, weight=self.norm_w,
                               post=post, bf16_copy=_tiles16(T, self.w_o))
         W = x.shape[1]

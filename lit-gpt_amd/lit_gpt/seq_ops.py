@@ -62,8 +62,8 @@ SIGNATURES = {
     "lgs_softcap": [_P, _L, _F, _P],
     "lgs_normattn_prepare": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P],
     "lgs_sinkattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P],
-    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
-    "lgs_gated_delta": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
+    "lgs_gated_delta": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
 }
 _RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
 
@@ -661,7 +661,8 @@ def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tenso
                   norm_eps: float = 1e-6):
     """qkv (T, 2 G d + H dv): q and k become unit vectors per head in place (q also times ``q_scale``). The raw decay
     inputs are the H d (``per_channel``) or H columns of ``a`` at ``a_off``, the raw betas the H columns of ``b`` at
-    ``b_off``. Returns (dec, beta): exp(-exp(A_log) softplus(a + dt_bias)) (T, H d) or (T, H), sigmoid(b) (T, H)."""
+    ``b_off``. Returns (dec, beta, kq): exp(-exp(A_log) softplus(a + dt_bias)) (T, H d) or (T, H), sigmoid(b) (T, H),
+    and k . q of the prepared vectors per key head (T, G)."""
     T, ld = qkv.shape
     n = H * d if per_channel else H
     if a.shape[0] != T or b.shape[0] != T or a_off + n > a.shape[1] or b_off + H > b.shape[1] or \
@@ -669,28 +670,30 @@ def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tenso
         raise ValueError("delta_prepare: shapes")
     dec = torch.empty(T, n, dtype=F32, device=qkv.device)
     beta = torch.empty(T, H, dtype=F32, device=qkv.device)
+    kq = torch.empty(T, G, dtype=F32, device=qkv.device)
     _check(load_library().lgs_delta_prepare(_dev(qkv, "qkv", F32), ld, _dev(a, "a", F32) + 4 * a_off, a.shape[1],
                                             _dev(b, "b", F32) + 4 * b_off, b.shape[1], _dev(A_log, "A_log", F32),
-                                            _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), beta.data_ptr(), T, H, G, d,
-                                            int(per_channel), float(q_scale), float(norm_eps), _stream()))
-    return dec, beta
+                                            _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), beta.data_ptr(),
+                                            kq.data_ptr(), T, H, G, d, int(per_channel), float(q_scale),
+                                            float(norm_eps), _stream()))
+    return dec, beta, kq
 
 
-def gated_delta(qkv: torch.Tensor, dec: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, seq_start: torch.Tensor,
-                seq_slot: torch.Tensor, seq_pos0: torch.Tensor, *, H: int, G: int, d: int, dv: int,
-                per_channel: bool, lanes: int = 0) -> torch.Tensor:
+def gated_delta(qkv: torch.Tensor, dec: torch.Tensor, beta: torch.Tensor, kq: torch.Tensor, state: torch.Tensor,
+                seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor, *, H: int, G: int, d: int,
+                dv: int, per_channel: bool, lanes: int = 0) -> torch.Tensor:
     """The gated delta rule over a packed batch, token by token: S <- diag(dec) S; u = beta (v - S^T k);
-    S <- S + k u^T; o = S^T q. qkv (T, 2 G d + H dv) prepared rows; state (slots, H, d, dv) fp32 is read unless a
-    sequence starts at position 0 and left at the step's last token. Returns o (T, H dv). ``lanes``: lanes that share
-    one state column (4, 8, 16; 0: chosen from the sizes)."""
+    S <- S + k u^T; o = S^T q. qkv (T, 2 G d + H dv) prepared rows, kq (T, G) their k . q (``delta_prepare``); state
+    (slots, H, d, dv) fp32 is read unless a sequence starts at position 0 and left at the step's last token. Returns
+    o (T, H dv). ``lanes``: lanes that share one state column (4, 8, 16; 0: chosen from the sizes)."""
     T, ld = qkv.shape
     B = seq_slot.numel()
     if ld != 2 * G * d + H * dv or tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or \
-            dec.shape != (T, H * d if per_channel else H) or beta.shape != (T, H):
+            dec.shape != (T, H * d if per_channel else H) or beta.shape != (T, H) or kq.shape != (T, G):
         raise ValueError("gated_delta: shapes")
     out = torch.empty(T, H * dv, dtype=F32, device=qkv.device)
     _check(load_library().lgs_gated_delta(_dev(qkv, "qkv", F32), ld, _dev(dec, "dec", F32), _dev(beta, "beta", F32),
-                                          _dev(state, "state", F32), _dev(seq_start, "seq_start", I32),
+                                          _dev(kq, "kq", F32), _dev(state, "state", F32), _dev(seq_start, "seq_start", I32),
                                           _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32),
                                           out.data_ptr(), B, H, G, d, dv, int(per_channel), int(lanes), _stream()))
     return out

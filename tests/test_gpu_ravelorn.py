@@ -400,7 +400,8 @@ def test_delta_rule_kernel_every_form(H, G, d, dv, lanes, per_channel):
     dec = torch.rand(T, H, d if per_channel else 1, generator=g) * 0.5 + 0.5
     qkv = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1).contiguous()
     sd = state.to(dev)
-    got = seq_ops.gated_delta(qkv.to(dev), dec.reshape(T, -1).contiguous().to(dev), beta.to(dev), sd, step.seq_start,
+    kq = (q * k).sum(-1)
+    got = seq_ops.gated_delta(qkv.to(dev), dec.reshape(T, -1).contiguous().to(dev), beta.to(dev), kq.to(dev), sd, step.seq_start,
                               step.seq_slot, step.seq_pos0, H=H, G=G, d=d, dv=dv, per_channel=per_channel, lanes=lanes)
     at = 0
     for s, p, n in zip(slots, first, lens):
@@ -429,17 +430,18 @@ def test_delta_prepare():
     b = torch.randn(T, H + 2, generator=g)
     A_log, bias = torch.randn(H, generator=g), torch.randn(H * d, generator=g)
     qd = qkv.to(dev)
-    dec, beta = seq_ops.delta_prepare(qd, a.to(dev), 3, b.to(dev), 2, A_log.to(dev), bias.to(dev), H=H, G=G, d=d,
-                                      per_channel=True, q_scale=0.25)
+    dec, beta, kq = seq_ops.delta_prepare(qd, a.to(dev), 3, b.to(dev), 2, A_log.to(dev), bias.to(dev), H=H, G=G, d=d,
+                                          per_channel=True, q_scale=0.25)
     x = qkv[:, :2 * G * d].double().view(T, 2 * G, d)
     want = x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
     want[:, :G] *= 0.25
     assert (qd[:, :2 * G * d].cpu().double().view(T, 2 * G, d) - want).abs().max() < 1e-6
     assert torch.equal(qd[:, 2 * G * d:].cpu(), qkv[:, 2 * G * d:])
+    assert (kq.cpu().double() - (want[:, :G] * want[:, G:]).sum(-1)).abs().max() < 1e-6
     wd = torch.exp(-torch.exp(A_log.double())[None, :, None] * orc.softplus(a[:, 3:].double() + bias.double()).view(T, H, d))
     assert (dec.cpu().double().view(T, H, d) - wd).abs().max() < 1e-6
     assert (beta.cpu().double() - torch.sigmoid(b[:, 2:].double())).abs().max() < 1e-6
-    dec1, _ = seq_ops.delta_prepare(qkv.to(dev), a.to(dev), 1, b.to(dev), 0, A_log.to(dev), bias[:H].contiguous().to(dev),
+    dec1, _, _ = seq_ops.delta_prepare(qkv.to(dev), a.to(dev), 1, b.to(dev), 0, A_log.to(dev), bias[:H].contiguous().to(dev),
                                     H=H, G=G, d=d, per_channel=False, q_scale=1.0)
     w1 = torch.exp(-torch.exp(A_log.double()) * orc.softplus(a[:, 1:1 + H].double() + bias[:H].double()))
     assert (dec1.cpu().double() - w1).abs().max() < 1e-6
