@@ -1,6 +1,7 @@
 /*
- * litgpt_seq.h — C ABI of liblitgpt_seq.so: the MI355X (gfx950) kernels of the layered models (retention and
- * latent-attention mixers, gated and sparse feed-forwards, per-layer token inputs) over an fp32 residual stream.
+ * litgpt_seq.h — C ABI of liblitgpt_seq.so: the MI355X (gfx950) kernels of the layered models (retention, latent-,
+ * differential- and sink-attention, state-space and delta-rule mixers, gated and sparse feed-forwards, per-layer token
+ * inputs) over an fp32 residual stream.
  *
  * Conventions: plain device pointers and sizes; every buffer is caller-owned; launches are asynchronous on `stream`
  * (graph-capturable); 0 on success, otherwise a hipError_t value with a message from lgs_last_error_string()
@@ -72,10 +73,11 @@ int lgs_retention(float* q, float* k, const float* v, long ld, float* state, con
                   int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked, float* ws, int max_chunks,
                   int T_rows, const int* pos, lgs_stream_t stream);
 /* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * weight[i] * act(g[t * ldg + h * dv + i]) * post
- * (weight: dv values shared by the heads, or NULL) */
+ * (weight: dv values shared by the heads, or NULL). With w_g2 ([H dv][rank], bf16 or fp32 with g2_f32) g holds the
+ * `rank` inner values of a low-rank gate per row and the gate's input is w_g2[h dv + i] . g[t * ldg ..]. */
 int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps, int act,
                   const float* weight, float post, void* o_bf16 /* optional rounded copy [T][H * dv] */,
-                  lgs_stream_t stream);
+                  const void* w_g2, int rank, int g2_f32, lgs_stream_t stream);
 /* latent attention, per token: c = rmsnorm(proj[kv_off .. + r]) * norm_w -> cache_c[slot][pos] (bf16, or fp32 with
  * cache_f32); rotary (pairs 2i, 2i + 1) of proj[kv_off + r .. + dr] -> cache_kr[slot][pos] (fp32); the rotated
  * part of every head's query (at q_off + h (d + dr) + d) is rotated in place. */
@@ -107,6 +109,10 @@ int lgs_moe_route(const float* z, long ld, int T, int E, int top, int* ids, floa
  * lowest index first among equals), wts = s at those places (not renormalised). E <= 256. */
 int lgs_moe_route_scores(const float* z, long ld, int T, int E, int top, const float* bias, int* ids, float* wts,
                          lgs_stream_t stream);
+/* the router product z = w h[t] (w [E][K], fp32 sums) and lgs_moe_route_scores' routing in one launch: the form of
+ * steps with few tokens */
+int lgs_moe_router(const float* h, long ldh, const void* w, int w_f32, int T, int K, int E, int top, const float* bias,
+                   int* ids, float* wts, lgs_stream_t stream);
 /* streaming experts: actbuf[t * top + k] = act(up[ids[t][k]] h[t]), or with gated (up holds per expert F gate rows,
  * then F up rows) act(gate h) * (up h); x[t] (+)= sum_k wts[t][k] down[ids[t][k]] actbuf[..]. An id >= n_real names
  * an identity expert without matrices: it is skipped by lgs_moe_up and contributes wts * hin[t] in lgs_moe_down. */
@@ -183,7 +189,18 @@ int lgs_sinkattn(const float* q, long ld, const void* cache_k, const void* cache
  * per_channel) or per head ([H]); kq[t][g] = k . q of the prepared vectors of key head g. */
 int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb, const float* A_log,
                       const float* dt_bias, float* dec, float* beta, float* kq, int T, int H, int G, int d,
-                      int per_channel, float q_scale, float norm_eps, lgs_stream_t stream);
+                      int per_channel, float q_scale, float norm_eps,
+                      const void* w_a2 /* optional: a holds `rank` values per row, the raw input of entry i is w_a2[i] . a */,
+                      int rank, int a2_f32, lgs_stream_t stream);
+/* The same for a step in which every sequence brings ONE token (row b of u belongs to sequence b), with the short
+ * causal convolution + silu of the C = 2 G d + H dv channels of u in the same launch: conv_w [C][taps] (column
+ * taps - 1 weights the token itself, no bias), conv_state [slots][taps - 1][C] as in lgs_conv_silu (read unless the
+ * sequence starts at position 0, shifted by one token). qkv [B][C] receives the prepared row. */
+int lgs_delta_step_prepare(const float* u, long ldu, const void* conv_w, int conv_f32, int taps, float* conv_state,
+                           const int* seq_slot, const int* seq_pos0, float* qkv, const float* a, long lda, const float* b,
+                           long ldb, const float* A_log, const float* dt_bias, float* dec, float* beta, float* kq, int B,
+                           int H, int G, int d, int dv, int per_channel, float q_scale, float norm_eps, const void* w_a2,
+                           int rank, int a2_f32, lgs_stream_t stream);
 /* Per sequence and head, token by token: S <- diag(dec) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q
  * (evaluated as S'^T q + u kq on the decayed state S', kq [T][G] = k . q from lgs_delta_prepare).
  * Head h reads q / k head h / (H / G). state [slots][H][d][dv] fp32 is read unless the sequence starts at position 0

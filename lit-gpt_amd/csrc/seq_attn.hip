@@ -1,18 +1,22 @@
-// Differential attention of the layered models: scores, weights and sums in fp32.
+// Softmax attention of the layered models over cached keys and values: scores, weights and sums in fp32.
 //
-// A query head carries two maps (q1, q2), a key head two key maps (k1, k2); both maps are softmax attentions over
-// the same values, combined as o = a1 - lambda a2, divided by the head's root mean square and scaled. Query head h
-// reads key/value head h / (H / G). Scores are (q . k) * scale, optionally soft-capped (cap * tanh(s / cap)); a
-// query at position i sees keys lo(i) <= j <= i with lo(i) = i - i % chunk for a chunked mask (chunks are aligned
-// to the sequence's position 0) and 0 without one.
+// Differential attention (two maps per head): a query head carries two maps (q1, q2), a key head two key maps
+// (k1, k2); both maps are softmax attentions over the same values, combined as o = a1 - lambda a2, divided by the
+// head's root mean square and scaled. Sink attention (one map per head): a plain softmax attention whose normaliser
+// also holds exp(sink) of the head. In both, query head h reads key/value head h / (H / G); scores are
+// (q . k) * scale, optionally soft-capped (cap * tanh(s / cap)); a query at position i sees keys lo(i) <= j <= i with
+// lo(i) = i - i % chunk for a chunked mask (chunks are aligned to the sequence's position 0) and 0 without one.
 //
 //   lgs_diffattn_prepare  per token: rotary (interleaved pairs 2i, 2i + 1 of the first rot_dims dims of every map)
 //                         on the queries in place and on the keys on their way into the cache; values into the cache.
 //                         Without key / value columns (a layer that reads another layer's cache) only the queries.
-//   lgs_diffattn          QT consecutive queries of one sequence and one head per workgroup against key tiles of 256
-//                         cached rows: a thread per key for the scores, an online softmax per (query, map), a thread
-//                         per value column for the weighted sums. One query per workgroup (decode) can spread its
-//                         keys over several workgroups, merged by a second launch.
+//   lgs_normattn_prepare  per token: queries divided by their root mean square and multiplied by a temperature that
+//                         grows with the position, in place; keys divided by their root mean square on their way
+//                         into the cache; values into the cache. No rotation.
+//   lgs_diffattn,         QT consecutive queries of one sequence and one head per workgroup (8 with two maps, 16 with
+//   lgs_sinkattn          one) against key tiles of 256 cached rows: a thread per key for the scores, an online
+//                         softmax per (query, map), a thread per value column for the weighted sums. One query per
+//                         workgroup (decode) can spread its keys over several workgroups, merged by a second launch.
 #include "seq_common.h"
 
 namespace lgs {

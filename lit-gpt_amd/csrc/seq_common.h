@@ -1,5 +1,6 @@
-// Shared declarations of liblitgpt_seq.so: the kernels of the layered models (retention and latent-attention
-// mixers, gated feed-forwards, sparse experts, per-layer token inputs) over an fp32 residual stream.
+// Shared declarations of liblitgpt_seq.so: the kernels of the layered models (retention, latent-, differential- and
+// sink-attention, state-space and delta-rule mixers, gated feed-forwards, sparse experts, per-layer token inputs) over
+// an fp32 residual stream.
 //
 // Conventions: activations are fp32 in memory in both precisions. A weight matrix is [out][in], either bf16 (raw
 // uint16; the activation operand of a product is then rounded to bf16 and the sum is fp32: the matrix-core
@@ -38,6 +39,36 @@ __device__ __forceinline__ float wload(const void* w, size_t i) {
 // the activation operand of a product: rounded to bf16 beside bf16 weights, as stored beside fp32 weights
 template <bool WF32>
 __device__ __forceinline__ float aop(float v) { return WF32 ? v : round_bf(v); }
+
+// eight consecutive weights starting at element i (i % 8 == 0, 16-byte aligned rows): one 16-byte load for bf16
+template <bool WF32>
+__device__ __forceinline__ void wload8(const void* w, size_t i, float* o) {
+  if (WF32) {
+    const float4 a = *(const float4*)((const float*)w + i), b = *(const float4*)((const float*)w + i + 4);
+    o[0] = a.x, o[1] = a.y, o[2] = a.z, o[3] = a.w, o[4] = b.x, o[5] = b.y, o[6] = b.z, o[7] = b.w;
+  } else {
+    const uint4 a = *(const uint4*)((const uint16_t*)w + i);
+    o[0] = bflo(a.x), o[1] = bfhi(a.x), o[2] = bflo(a.y), o[3] = bfhi(a.y);
+    o[4] = bflo(a.z), o[5] = bfhi(a.z), o[6] = bflo(a.w), o[7] = bfhi(a.w);
+  }
+}
+// the product of one row of a small second map with its `rank` inputs x (already rounded as the weights' precision
+// asks, in LDS or registers' reach): w row i holds rank weights; rank % 8 == 0 takes 16-byte loads
+template <bool WF32>
+__device__ __forceinline__ float lowrank_dot(const void* w, size_t i, const float* x, int rank) {
+  float acc = 0.0f;
+  if ((rank & 7) == 0) {
+    for (int r = 0; r < rank; r += 8) {
+      float u[8];
+      wload8<WF32>(w, i * rank + r, u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc = fmaf(x[r + e], u[e], acc);
+    }
+  } else {
+    for (int r = 0; r < rank; ++r) acc = fmaf(x[r], wload<WF32>(w, i * rank + r), acc);
+  }
+  return acc;
+}
 
 // sum over the 256 threads of a workgroup (4 waves); `red` holds 4 floats; every thread gets the sum
 __device__ __forceinline__ float block_sum_256(float v, float* red) {

@@ -6,6 +6,8 @@
 //
 //   lgs_delta_prepare   per token: q and k (after their convolution) become unit vectors per head, q times q_scale;
 //                       beta = sigmoid(raw); g = exp(-exp(A_log) softplus(raw + dt_bias)); k . q per key head
+//   lgs_delta_step_prepare  the same for a step in which every sequence brings one token, with the short convolution
+//                       of q | k | v (and the shift of its stored inputs) in the same launch
 //   lgs_gated_delta     the recurrence, token by token for every step kind. The columns of S never mix, so a column
 //                       is owned by LPC adjacent lanes that hold d / LPC of its rows in registers; the two dot
 //                       products over the rows (both against the decayed state: o = S'^T q + u (k . q)) are summed
@@ -31,15 +33,33 @@ struct DeltaPrepArgs {
   float* kq;                     // [T][G]: k . q of the prepared vectors
   int H, G, d, per_channel;
   float q_scale, norm_eps;
+  // optional second map of a low-rank decay input: a holds `rank` values per row and the raw input of entry i is
+  // w_a2[i] . a (w_a2 [H d or H][rank], bf16 or fp32)
+  const void* w_a2;
+  int rank, a2_f32;
+  // the fused one-token form only: the convolution's inputs u [B][ldu] (C = 2 G d + H dv channels), its weights
+  // [C][taps] and its slot-indexed history [slots][taps - 1][C]
+  const float* u;
+  long ldu;
+  const void* conv_w;
+  int conv_f32, taps, C;
+  float* conv_state;
+  const int *seq_slot, *seq_pos0;
 };
 
-// grid (T): wave w makes the vectors w, w + 4, ... of the 2 G query / key heads unit vectors; all threads walk the
-// decays and betas
-__global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
-  const size_t t = blockIdx.x;
+// One row's preparation by a whole workgroup: wave w makes the vectors w, w + 4, ... of the 2 G query / key heads
+// unit vectors; all threads walk the decays and betas; then k . q per key head.
+constexpr int kMaxRank = 512;  // inner size of a low-rank second map that is folded into a consuming kernel
+
+template <bool A2F32>
+__device__ __forceinline__ void delta_prepare_row(const DeltaPrepArgs& p, size_t t) {
+  __shared__ float a1[kMaxRank];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int d = p.d;
   float* row = p.qkv + t * p.ld;
+  if (p.w_a2)
+    for (int r = threadIdx.x; r < p.rank; r += 256) a1[r] = aop<A2F32>(p.a[t * p.lda + r]);
+  __syncthreads();
   for (int vec = wave; vec < 2 * p.G; vec += 4) {
     float* x = row + (size_t)vec * d;
     float ss = 0.0f;
@@ -51,7 +71,8 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
   const int dc = p.per_channel ? d : 1, n = p.H * dc;
   for (int i = threadIdx.x; i < n; i += 256) {
     const float rate = expf(p.A_log[i / dc]);
-    p.dec[t * n + i] = expf(-rate * softplus_d(p.a[t * p.lda + i] + p.dt_bias[i]));
+    const float raw = p.w_a2 ? lowrank_dot<A2F32>(p.w_a2, i, a1, p.rank) : p.a[t * p.lda + i];
+    p.dec[t * n + i] = expf(-rate * softplus_d(raw + p.dt_bias[i]));
   }
   for (int h = threadIdx.x; h < p.H; h += 256) p.beta[t * p.H + h] = sigmoid_f(p.b[t * p.ldb + h]);
   __syncthreads();  // the unit vectors of all heads are written
@@ -61,6 +82,87 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
     for (int i = lane; i < d; i += 64) s = fmaf(q[i], k[i], s);
     s = wave_sum(s);
     if (lane == 0) p.kq[t * p.G + g] = s;
+  }
+}
+
+// grid (T)
+template <bool A2F32>
+__global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
+  delta_prepare_row<A2F32>(p, blockIdx.x);
+}
+
+// One channel of the short convolution for a one-token step: the weighted sum of the token's input and the slot's
+// stored inputs (zeros before the sequence's start), which are shifted by one; returns silu of the sum.
+template <bool WF32>
+__device__ __forceinline__ float conv_step_channel(const DeltaPrepArgs& p, int b, int c, int pos0, float* st) {
+  const int taps = p.taps, hist = taps - 1, C = p.C;
+  const float cur = p.u[(size_t)b * p.ldu + c];
+  float acc = wload<WF32>(p.conv_w, (size_t)c * taps + hist) * cur;
+  float prev = cur;  // walks the history from the newest stored input to the oldest, shifting it on the way
+  for (int j = hist - 1; j >= 0; --j) {
+    const float x = pos0 - (hist - j) >= 0 ? st[(size_t)j * C + c] : 0.0f;
+    acc = fmaf(wload<WF32>(p.conv_w, (size_t)c * taps + j), x, acc);
+    st[(size_t)j * C + c] = prev;
+    prev = x;
+  }
+  return acc / (1.0f + expf(-acc));
+}
+
+// The one-token step (every sequence brings one token; row b belongs to sequence b): convolution + silu of the
+// token's q | k | v channels and the row's preparation in one launch. grid (B, G + ceil(H dv / 256) + ceil(n / 256)):
+// workgroup y < G convolves and normalises q and k of key head y and leaves their k . q; the next ones convolve 256
+// value channels each; the last ones make 256 decays each (the first of them also the betas).
+template <bool WF32, bool A2F32>
+__global__ void __launch_bounds__(256) delta_step_prepare_kernel(DeltaPrepArgs p) {
+  __shared__ float buf[2 * 512];
+  __shared__ float red[4];
+  const int b = blockIdx.x, y = blockIdx.y, tid = threadIdx.x;
+  const int d = p.d, G = p.G, C = p.C, hist = p.taps - 1;
+  const int pos0 = p.seq_pos0[b];
+  float* st = p.conv_state + (size_t)p.seq_slot[b] * max(hist, 1) * C;
+  float* row = p.qkv + (size_t)b * p.ld;
+  const int nv = C - 2 * G * d, parts_v = (nv + 255) / 256;
+  if (y < G) {
+    for (int i = tid; i < 2 * d; i += 256) {
+      const int c = i < d ? y * d + i : (G + y) * d + (i - d);
+      buf[i] = conv_step_channel<WF32>(p, b, c, pos0, st);
+    }
+    __syncthreads();
+    float sq = 0.0f, sk = 0.0f;
+    for (int i = tid; i < d; i += 256) {
+      sq = fmaf(buf[i], buf[i], sq);
+      sk = fmaf(buf[d + i], buf[d + i], sk);
+    }
+    sq = block_sum_256(sq, red);
+    sk = block_sum_256(sk, red);
+    const float fq = p.q_scale / sqrtf(sq + p.norm_eps), fk = 1.0f / sqrtf(sk + p.norm_eps);
+    float kq = 0.0f;
+    for (int i = tid; i < d; i += 256) {
+      const float qn = buf[i] * fq, kn = buf[d + i] * fk;
+      row[(size_t)y * d + i] = qn;
+      row[(size_t)(G + y) * d + i] = kn;
+      kq = fmaf(qn, kn, kq);
+    }
+    kq = block_sum_256(kq, red);
+    if (tid == 0) p.kq[(size_t)b * G + y] = kq;
+  } else if (y < G + parts_v) {
+    const int c = 2 * G * d + (y - G) * 256 + tid;
+    if (c < C) row[c] = conv_step_channel<WF32>(p, b, c, pos0, st);
+  } else {
+    const int blk = y - G - parts_v;
+    const int dc = p.per_channel ? d : 1, n = p.H * dc;
+    if (p.w_a2) {
+      for (int r = tid; r < p.rank; r += 256) buf[r] = aop<A2F32>(p.a[(size_t)b * p.lda + r]);
+      __syncthreads();
+    }
+    const int i = blk * 256 + tid;
+    if (i < n) {
+      const float rate = expf(p.A_log[i / dc]);
+      const float raw = p.w_a2 ? lowrank_dot<A2F32>(p.w_a2, i, buf, p.rank) : p.a[(size_t)b * p.lda + i];
+      p.dec[(size_t)b * n + i] = expf(-rate * softplus_d(raw + p.dt_bias[i]));
+    }
+    if (blk == 0)
+      for (int h = tid; h < p.H; h += 256) p.beta[(size_t)b * p.H + h] = sigmoid_f(p.b[(size_t)b * p.ldb + h]);
   }
 }
 
@@ -260,13 +362,45 @@ static bool gated_delta_launch(DeltaArgs p, int B, hipStream_t stream) {
 
 extern "C" int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb,
                                  const float* A_log, const float* dt_bias, float* dec, float* beta, float* kq, int T,
-                                 int H, int G, int d, int per_channel, float q_scale, float norm_eps,
-                                 hipStream_t stream) {
+                                 int H, int G, int d, int per_channel, float q_scale, float norm_eps, const void* w_a2,
+                                 int rank, int a2_f32, hipStream_t stream) {
   LGA_CHECK_ARG(qkv && a && b && A_log && dt_bias && dec && beta && kq && T > 0, "lgs_delta_prepare: bad arguments");
   LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && ld >= 2L * G * d, "lgs_delta_prepare: bad sizes");
+  LGA_CHECK_ARG(!w_a2 || (rank > 0 && rank <= lgs::kMaxRank), "lgs_delta_prepare: inner size of the decay map 1..512");
   lgs::DeltaPrepArgs p{qkv, ld, a, lda, b, ldb, A_log, dt_bias, dec, beta, kq, H, G, d, per_channel ? 1 : 0, q_scale,
-                       norm_eps};
-  lgs::delta_prepare_kernel<<<T, 256, 0, stream>>>(p);
+                       norm_eps, w_a2, rank, a2_f32, nullptr, 0, nullptr, 0, 0, 0, nullptr, nullptr, nullptr};
+  if (a2_f32) lgs::delta_prepare_kernel<true><<<T, 256, 0, stream>>>(p);
+  else lgs::delta_prepare_kernel<false><<<T, 256, 0, stream>>>(p);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_delta_step_prepare(const float* u, long ldu, const void* conv_w, int conv_f32, int taps,
+                                      float* conv_state, const int* seq_slot, const int* seq_pos0, float* qkv,
+                                      const float* a, long lda, const float* b, long ldb, const float* A_log,
+                                      const float* dt_bias, float* dec, float* beta, float* kq, int B, int H, int G,
+                                      int d, int dv, int per_channel, float q_scale, float norm_eps, const void* w_a2,
+                                      int rank, int a2_f32, hipStream_t stream) {
+  LGA_CHECK_ARG(u && conv_w && conv_state && seq_slot && seq_pos0 && qkv && a && b && A_log && dt_bias && dec && beta &&
+                    kq && B > 0,
+                "lgs_delta_step_prepare: bad arguments");
+  LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && taps >= 1 && taps <= 16,
+                "lgs_delta_step_prepare: bad sizes (taps 1..16)");
+  LGA_CHECK_ARG(!w_a2 || (rank > 0 && rank <= lgs::kMaxRank),
+                "lgs_delta_step_prepare: inner size of the decay map 1..512");
+  const int C = 2 * G * d + H * dv;
+  LGA_CHECK_ARG(ldu >= C, "lgs_delta_step_prepare: channels outside the row");
+  lgs::DeltaPrepArgs p{qkv, C, a, lda, b, ldb, A_log, dt_bias, dec, beta, kq, H, G, d, per_channel ? 1 : 0, q_scale,
+                       norm_eps, w_a2, rank, a2_f32, u, ldu, conv_w, conv_f32, taps, C, conv_state, seq_slot, seq_pos0};
+  const int n = per_channel ? H * d : H;
+  const dim3 grid(B, G + (H * dv + 255) / 256 + (n + 255) / 256);
+  LGA_CHECK_ARG(d <= 512 && grid.y <= 65535, "lgs_delta_step_prepare: key dim <= 512");
+  if (conv_f32) {
+    if (a2_f32) lgs::delta_step_prepare_kernel<true, true><<<grid, 256, 0, stream>>>(p);
+    else lgs::delta_step_prepare_kernel<true, false><<<grid, 256, 0, stream>>>(p);
+  } else {
+    if (a2_f32) lgs::delta_step_prepare_kernel<false, true><<<grid, 256, 0, stream>>>(p);
+    else lgs::delta_step_prepare_kernel<false, false><<<grid, 256, 0, stream>>>(p);
+  }
   LGA_LAUNCH_RETURN();
 }
 

@@ -16,18 +16,6 @@
 
 namespace lgs {
 
-// eight consecutive weights starting at element i (i % 8 == 0, 16-byte aligned rows): one 16-byte load for bf16
-template <bool WF32>
-__device__ __forceinline__ void wload8(const void* w, size_t i, float* o) {
-  if (WF32) {
-    const float4 a = *(const float4*)((const float*)w + i), b = *(const float4*)((const float*)w + i + 4);
-    o[0] = a.x, o[1] = a.y, o[2] = a.z, o[3] = a.w, o[4] = b.x, o[5] = b.y, o[6] = b.z, o[7] = b.w;
-  } else {
-    const uint4 a = *(const uint4*)((const uint16_t*)w + i);
-    o[0] = bflo(a.x), o[1] = bfhi(a.x), o[2] = bflo(a.y), o[3] = bfhi(a.y);
-    o[4] = bflo(a.z), o[5] = bfhi(a.z), o[6] = bflo(a.w), o[7] = bfhi(a.w);
-  }
-}
 // the dot products of one activation row (fp32, rounded as the weights' precision asks) with two weight rows of n
 // elements; `vec` (n % 8 == 0 and 16-byte aligned rows) takes 16-byte loads
 template <bool WF32>
@@ -132,16 +120,15 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__
     for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= den;
 }
 
-// one wave per token: s = softmax(z) over all E outputs; the `top` largest of s + bias (lowest index first among
-// equals) are chosen, and their weights are s itself: not renormalised, without the bias
-__global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* __restrict__ z, long ld, int E, int top,
-                                                              const float* __restrict__ bias, int* __restrict__ ids,
-                                                              float* __restrict__ wts) {
-  const int t = blockIdx.x, lane = threadIdx.x;
+// one wave: s = softmax(z) over all E outputs (z: the token's router logits, global or LDS); the `top` largest of
+// s + bias (lowest index first among equals) are chosen, and their weights are s itself: not renormalised, without
+// the bias
+__device__ __forceinline__ void route_scores_wave(const float* z, int E, int top, const float* __restrict__ bias,
+                                                  int* __restrict__ ids, float* __restrict__ wts, int lane) {
   float s[4], c[4], mx = -INFINITY;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    s[e] = lane + 64 * e < E ? z[(size_t)t * ld + lane + 64 * e] : -INFINITY;
+    s[e] = lane + 64 * e < E ? z[lane + 64 * e] : -INFINITY;
     mx = fmaxf(mx, s[e]);
   }
   mx = wave_max(mx);
@@ -181,13 +168,41 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* __res
       }
     }
     if (lane == 0) {
-      ids[(size_t)t * top + k] = bi;
-      wts[(size_t)t * top + k] = bs;
+      ids[k] = bi;
+      wts[k] = bs;
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (lane + 64 * e == bi) c[e] = -INFINITY;
   }
+}
+
+__global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* __restrict__ z, long ld, int E, int top,
+                                                              const float* __restrict__ bias, int* __restrict__ ids,
+                                                              float* __restrict__ wts) {
+  const size_t t = blockIdx.x;
+  route_scores_wave(z + t * ld, E, top, bias, ids + t * top, wts + t * top, threadIdx.x);
+}
+
+// grid (T), 1024 threads: the router's logits of one token (wave w takes outputs w, w + 16, ...; fp32 sums, the
+// operand rounded as the weights' precision asks, 16-byte weight loads where the rows allow) and the routing above,
+// in one launch: the form of steps with few tokens
+template <bool WF32>
+__global__ void __launch_bounds__(1024) moe_router_kernel(const float* __restrict__ h, long ldh, const void* __restrict__ w,
+                                                          int K, int E, int top, const float* __restrict__ bias,
+                                                          int* __restrict__ ids, float* __restrict__ wts) {
+  __shared__ float z[256];
+  const size_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float* x = h + t * ldh;
+  const bool vec = (K & 7) == 0 && (ldh & 3) == 0 && ((uintptr_t)h & 15) == 0;
+  for (int e = wave; e < E; e += 16) {
+    float a0, a1;
+    dot2<WF32>(x, w, (size_t)e * K, (size_t)e * K, K, vec, lane, a0, a1);
+    if (lane == 0) z[e] = a0;
+  }
+  __syncthreads();
+  if (wave == 0) route_scores_wave(z, E, top, bias, ids + t * top, wts + t * top, lane);
 }
 
 // grid (ceil(F / 8), pairs): pair = token * top + choice; act[pair][f] = act(up_e[f] . h_token); GATED: an expert's
@@ -392,6 +407,15 @@ extern "C" int lgs_moe_route_scores(const float* z, long ld, int T, int E, int t
   LGA_CHECK_ARG(E > 0 && E <= 256 && top > 0 && top <= E,
                 "lgs_moe_route_scores: experts must be <= 256 and top <= experts");
   lgs::moe_route_scores_kernel<<<T, 64, 0, stream>>>(z, ld, E, top, bias, ids, wts);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_moe_router(const float* h, long ldh, const void* w, int w_f32, int T, int K, int E, int top,
+                              const float* bias, int* ids, float* wts, hipStream_t stream) {
+  LGA_CHECK_ARG(h && w && ids && wts && T > 0 && K > 0 && ldh >= K, "lgs_moe_router: bad arguments");
+  LGA_CHECK_ARG(E > 0 && E <= 256 && top > 0 && top <= E, "lgs_moe_router: experts must be <= 256 and top <= experts");
+  if (w_f32) lgs::moe_router_kernel<true><<<T, 1024, 0, stream>>>(h, ldh, w, K, E, top, bias, ids, wts);
+  else lgs::moe_router_kernel<false><<<T, 1024, 0, stream>>>(h, ldh, w, K, E, top, bias, ids, wts);
   LGA_LAUNCH_RETURN();
 }
 

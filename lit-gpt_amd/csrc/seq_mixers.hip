@@ -301,15 +301,23 @@ static size_t retention_chunk_lds(int d) {
 
 // grid (T, H): o[t][h][:] <- (unit ? o / rms(o) : o) * w[:] * act(g[t * ldg + h * dv + :]) * post
 // (w: optional weight shared by the heads; o16: optional rounded copy, the operand of the out-projection's bf16
-// MFMA tiles)
+// MFMA tiles). With w_g2 ([H dv][rank], bf16 or fp32) the gate's input is the second map of a low-rank gate:
+// g holds `rank` values per row and entry i's input is w_g2[i] . g.
+template <bool G2F32>
 __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, const float* __restrict__ g, long ldg,
                                                         int H, int dv, int unit, float eps, int act,
                                                         const float* __restrict__ w, float post,
-                                                        uint16_t* __restrict__ o16) {
+                                                        uint16_t* __restrict__ o16, const void* __restrict__ w_g2,
+                                                        int rank) {
   __shared__ float red[4];
+  __shared__ float g1[512];
   const int t = blockIdx.x, h = blockIdx.y;
   float* orow = o + ((size_t)t * H + h) * dv;
   const float* grow = g + (size_t)t * ldg + (size_t)h * dv;
+  if (w_g2) {
+    for (int r = threadIdx.x; r < rank; r += 256) g1[r] = aop<G2F32>(g[(size_t)t * ldg + r]);
+    __syncthreads();
+  }
   float rstd = 1.0f;
   if (unit) {
     float ss = 0.0f;
@@ -320,7 +328,8 @@ __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, c
   for (int i = threadIdx.x; i < dv; i += 256) {
     float v = orow[i] * rstd;
     if (w) v *= w[i];
-    v *= act_f(act, grow[i]);
+    const float gin = w_g2 ? lowrank_dot<G2F32>(w_g2, (size_t)h * dv + i, g1, rank) : grow[i];
+    v *= act_f(act, gin);
     if (post != 1.0f) v *= post;
     orow[i] = v;
     if (o16) o16[((size_t)t * H + h) * dv + i] = f2bf(v);
@@ -857,10 +866,16 @@ extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float*
 }
 
 extern "C" int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps,
-                             int act, const float* weight, float post, void* o_bf16, hipStream_t stream) {
-  LGA_CHECK_ARG(o && g && T > 0 && H > 0 && H <= 65535 && dv > 0, "lgs_head_gate: bad arguments");
-  lgs::head_gate_kernel<<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act, weight, post,
-                                                        (uint16_t*)o_bf16);
+                             int act, const float* weight, float post, void* o_bf16, const void* w_g2, int rank,
+                             int g2_f32, hipStream_t stream) {
+  LGA_CHECK_ARG(o && g && T > 0 && H > 0 && H <= 65535 && dv > 0 && (!w_g2 || (rank > 0 && rank <= 512)),
+                "lgs_head_gate: bad arguments (inner size of a low-rank gate 1..512)");
+  if (g2_f32)
+    lgs::head_gate_kernel<true><<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act, weight, post,
+                                                                (uint16_t*)o_bf16, w_g2, rank);
+  else
+    lgs::head_gate_kernel<false><<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act, weight, post,
+                                                                 (uint16_t*)o_bf16, w_g2, rank);
   LGA_LAUNCH_RETURN();
 }
 

@@ -180,8 +180,10 @@ class PostSublayer(nn.Module):
     def forward(self, x: torch.Tensor, x16: Optional[torch.Tensor], step: StepBatch, cache) -> torch.Tensor:
         """x (T, width): the residual (x16: its bf16 copy for the MFMA tiles). Returns the sublayer's output, unnormed."""
         n_in, W = self.w_in.shape
-        proj = torch.empty(step.T, n_in, dtype=torch.float32, device=x.device)
-        seq_ops.linear(x if x16 is None else x16, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
+        proj = None
+        if self.module.wants_proj(step.T):
+            proj = torch.empty(step.T, n_in, dtype=torch.float32, device=x.device)
+            seq_ops.linear(x if x16 is None else x16, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
         y = torch.empty(step.T, W, dtype=torch.float32, device=x.device)
         if cache is None:
             self.module(proj, x, y, h16=x16, accumulate=False)

@@ -6,6 +6,10 @@ gate and up matrices, the router), and each module finds its columns in the resu
 module's rows of that matrix, ``bind`` tells it where they landed. Outputs are accumulated into the fp32 residual
 stream ``x`` by the epilogue of the out-projection (or the expert combine), so a layer needs no add kernel.
 
+Mixers here: ``Retention``, ``LatentAttention``, ``DiffAttention``, ``SelectiveScan``, ``GatedDelta`` (the gated delta
+rule with a decay per head or per head and key channel), ``SinkAttention`` (unit-RMS queries and keys, a query
+temperature, a sink in the normaliser) and ``ParallelMixer`` (the last two side by side on one input projection).
+
 A step is a packed batch (``StepBatch``): the tokens of all sequences row after row, with per-token cache slot and
 position and per-sequence row range, slot and first position, all int32 on the device. Sizes, decays, scales, rotary
 dims / bases and layouts are constructor parameters; nothing is fixed to one model.
@@ -76,6 +80,10 @@ class InputReader(nn.Module):
 
     def bind(self, offsets: Dict[str, int]) -> None:
         self.off = dict(offsets)
+
+    def wants_proj(self, rows: int) -> bool:
+        """Whether a step of ``rows`` tokens needs the shared input projection made for this module."""
+        return True
 
 
 class Retention(InputReader):
@@ -286,6 +294,8 @@ class GatedDelta(InputReader):
     is divided by its root mean square, times a weight shared by the heads, times the gate, then projected. The state
     (S and the convolution's last taps - 1 inputs) lives in a cache slot."""
 
+    FUSED_ROWS = 8  # one-token steps of up to this many sequences take the fused convolution + preparation launch
+
     def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype,
                  per_channel: Optional[bool] = None) -> None:
         super().__init__()
@@ -328,23 +338,36 @@ class GatedDelta(InputReader):
         H, G, d, dv = self.H, self.G, self.d, self.dv
         T, ld = proj.shape
         tables = (step.seq_start, step.seq_slot, step.seq_pos0)
-        qkv = seq_ops.conv_silu(proj, self.off["qkv"], self.conv_w, self.conv_b, cache.conv, *tables,
-                                step.max_len or T)
-        if self.per_channel:
-            ra, rg = self.w_a2.shape[1], self.w_g2.shape[1]
-            a = torch.empty(T, H * d, dtype=torch.float32, device=proj.device)
-            seq_ops.linear(proj, self.w_a2, M=T, N=H * d, K=ra, y=a, a_off=self.off["a1"], lda=ld, ldy=H * d)
-            gate = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
-            seq_ops.linear(proj, self.w_g2, M=T, N=H * dv, K=rg, y=gate, a_off=self.off["g1"], lda=ld, ldy=H * dv)
-            a_off, g_off, act = 0, 0, seq_ops.ACT_SIGMOID
+        kw = dict(H=H, G=G, d=d, per_channel=self.per_channel, q_scale=float(d) ** -0.5)
+        if step.max_len == 1 and T <= self.FUSED_ROWS and (not self.per_channel or
+                                                           max(self.w_a2.shape[1], self.w_g2.shape[1]) <= 512):
+            # one token per sequence (decode): convolution + preparation in one launch, and the second maps of the
+            # low-rank decay and gate inside the kernels that consume them
+            a_off = self.off["a1"] if self.per_channel else self.off["a"]
+            w2 = (self.w_a2, self.w_g2) if self.per_channel else (None, None)
+            qkv, dec, beta, kq = seq_ops.delta_step_prepare(proj, self.off["qkv"], self.conv_w, cache.conv, step.seq_slot,
+                                                            step.seq_pos0, a_off, self.off["b"], self.A_log,
+                                                            self.dt_bias, dv=dv, w_a2=w2[0], **kw)
+            gate, g_off, g2 = proj, (self.off["g1"] if self.per_channel else self.off["g"]), w2[1]
         else:
-            a, a_off, gate, g_off, act = proj, self.off["a"], proj, self.off["g"], seq_ops.ACT_SILU
-        dec, beta, kq = seq_ops.delta_prepare(qkv, a, a_off, proj, self.off["b"], self.A_log, self.dt_bias, H=H, G=G, d=d,
-                                              per_channel=self.per_channel, q_scale=float(d) ** -0.5)
+            qkv = seq_ops.conv_silu(proj, self.off["qkv"], self.conv_w, self.conv_b, cache.conv, *tables,
+                                    step.max_len or T)
+            if self.per_channel:
+                ra, rg = self.w_a2.shape[1], self.w_g2.shape[1]
+                a = torch.empty(T, H * d, dtype=torch.float32, device=proj.device)
+                seq_ops.linear(proj, self.w_a2, M=T, N=H * d, K=ra, y=a, a_off=self.off["a1"], lda=ld, ldy=H * d)
+                gate = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
+                seq_ops.linear(proj, self.w_g2, M=T, N=H * dv, K=rg, y=gate, a_off=self.off["g1"], lda=ld, ldy=H * dv)
+                a_off, g_off = 0, 0
+            else:
+                a, a_off, gate, g_off = proj, self.off["a"], proj, self.off["g"]
+            g2 = None
+            dec, beta, kq = seq_ops.delta_prepare(qkv, a, a_off, proj, self.off["b"], self.A_log, self.dt_bias, **kw)
         o = seq_ops.gated_delta(qkv, dec, beta, kq, cache.s, *tables, H=H, G=G, d=d, dv=dv,
                                 per_channel=self.per_channel)
+        act = seq_ops.ACT_SIGMOID if self.per_channel else seq_ops.ACT_SILU
         o = seq_ops.head_gate(o, gate, g_off, H=H, dv=dv, unit_norm=True, eps=self.eps, act=act, weight=self.norm_w,
-                              post=post, bf16_copy=_tiles16(T, self.w_o))
+                              post=post, bf16_copy=_tiles16(T, self.w_o), w_g2=g2)
         W = x.shape[1]
         seq_ops.linear(o, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
 
@@ -505,6 +528,8 @@ class SparseFeedForward(InputReader):
             raise ValueError("mlp experts: unexpected shapes")
         self.register_buffer("w_up", up.to(device=device, dtype=dtype).contiguous())  # gated: gate rows, then up rows
         self.register_buffer("w_down", down.to(device=device, dtype=dtype).contiguous())
+        # (steps with few tokens compute the router's logits inside the routing launch, from this copy)
+        self.register_buffer("w_router", w["router"].to(device=device, dtype=dtype).contiguous() if self.gated else None)
         self.register_buffer("correction", None)
         if self.gated and "correction" in w:
             if w["correction"].numel() != self.n_router:
@@ -514,12 +539,19 @@ class SparseFeedForward(InputReader):
     def in_parts(self):
         return self._in
 
-    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor, h16: Optional[torch.Tensor] = None,
-                accumulate: bool = True) -> None:
-        """h: the sublayer's input (fp32); h16: its bf16 copy when the layer made one (the grouped products read it)."""
+    def wants_proj(self, rows: int) -> bool:
+        """Whether a step of ``rows`` tokens needs the layer's input projection (the router logits) made for it."""
+        return not (self.gated and rows * self.top <= self.STREAM_PAIRS)
+
+    def forward(self, proj: Optional[torch.Tensor], h: torch.Tensor, x: torch.Tensor,
+                h16: Optional[torch.Tensor] = None, accumulate: bool = True) -> None:
+        """h: the sublayer's input (fp32); h16: its bf16 copy when the layer made one (the grouped products read it).
+        ``proj`` None (score routing, few tokens): the router's logits are made inside the routing launch."""
         T, W = h.shape
         E, top, F = self.E, self.top, self.ff
-        if self.gated:
+        if self.gated and proj is None:
+            ids, wts = seq_ops.moe_router(h, self.w_router, top, self.correction)
+        elif self.gated:
             ids, wts = seq_ops.moe_route_scores(proj, self.off["router"], self.n_router, top, self.correction)
         else:
             ids, wts = seq_ops.moe_route(proj, self.off["router"], E, top)

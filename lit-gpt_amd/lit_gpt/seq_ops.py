@@ -36,13 +36,14 @@ SIGNATURES = {
     "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P, _P],
     "lgs_gather_rows": [_P, _P, _P, _I, _I, _P],
     "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _P],
-    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P, _F, _P, _P],
+    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P, _F, _P, _P, _I, _I, _P],
     "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
     "lgs_latent_attention_tiles": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _I, _P],
     "lgs_moe_route": [_P, _L, _I, _I, _I, _P, _P, _P],
     "lgs_moe_route_scores": [_P, _L, _I, _I, _I, _P, _P, _P, _P],
+    "lgs_moe_router": [_P, _L, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
     "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _L, _I, _P],
     "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
@@ -62,7 +63,9 @@ SIGNATURES = {
     "lgs_softcap": [_P, _L, _F, _P],
     "lgs_normattn_prepare": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P],
     "lgs_sinkattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P],
-    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
+    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P, _I, _I, _P],
+    "lgs_delta_step_prepare": [_P, _L, _P, _I, _I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
+                               _I, _F, _F, _P, _I, _I, _P],
     "lgs_gated_delta": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
 }
 _RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
@@ -222,17 +225,22 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: tor
 
 def head_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, *, H: int, dv: int, unit_norm: bool, eps: float,
               act: int, bf16_copy: bool = False, weight: Optional[torch.Tensor] = None,
-              post: float = 1.0) -> torch.Tensor:
+              post: float = 1.0, w_g2: Optional[torch.Tensor] = None) -> torch.Tensor:
     """In place on o (T, H * dv): per head optional unit RMS, times ``weight`` (dv values shared by the heads), times
-    act(gate), the gate at proj[:, g_off:], times ``post``. Returns o, or with ``bf16_copy`` its rounding to bf16
-    (the operand of a bf16 MFMA product)."""
+    act(gate), the gate at proj[:, g_off:], times ``post``. With ``w_g2`` (H dv, rank) the columns of ``proj`` at
+    ``g_off`` are the rank inner values of a low-rank gate and the gate's input is w_g2 times them (the form of steps
+    with few tokens). Returns o, or with ``bf16_copy`` its rounding to bf16 (the operand of a bf16 MFMA product)."""
     T, ld = proj.shape
-    if o.shape != (T, H * dv) or g_off + H * dv > ld or (weight is not None and weight.numel() != dv):
+    cols = H * dv if w_g2 is None else w_g2.shape[1]
+    if o.shape != (T, H * dv) or g_off + cols > ld or (weight is not None and weight.numel() != dv) or \
+            (w_g2 is not None and w_g2.shape[0] != H * dv):
         raise ValueError("head_gate: shapes")
     o16 = torch.empty(T, H * dv, dtype=torch.bfloat16, device=o.device) if bf16_copy else None
     _check(load_library().lgs_head_gate(_dev(o, "o", F32), _dev(proj, "proj", F32) + 4 * g_off, ld, T, H, dv,
                                         int(unit_norm), float(eps), act, _opt(weight, "weight", F32), float(post),
-                                        _opt(o16, "o_bf16", torch.bfloat16), _stream()))
+                                        _opt(o16, "o_bf16", torch.bfloat16), _opt(w_g2, "w_g2"),
+                                        0 if w_g2 is None else w_g2.shape[1], 0 if w_g2 is None else _wf32(w_g2, "w_g2"),
+                                        _stream()))
     return o16 if bf16_copy else o
 
 
@@ -327,6 +335,19 @@ def moe_route_scores(proj: torch.Tensor, z_off: int, E: int, top: int, bias: Opt
     wts = torch.empty(T, top, dtype=F32, device=proj.device)
     _check(load_library().lgs_moe_route_scores(_dev(proj, "proj", F32) + 4 * z_off, ld, T, E, top,
                                                _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), _stream()))
+    return ids, wts
+
+
+def moe_router(h: torch.Tensor, w: torch.Tensor, top: int, bias: Optional[torch.Tensor] = None):
+    """``moe_route_scores`` of the router logits w h, both in one launch (steps with few tokens). w (E, K)."""
+    T, K = h.shape
+    E = w.shape[0]
+    if w.shape[1] != K or (bias is not None and bias.numel() != E):
+        raise ValueError("moe_router: shapes")
+    ids = torch.empty(T, top, dtype=I32, device=h.device)
+    wts = torch.empty(T, top, dtype=F32, device=h.device)
+    _check(load_library().lgs_moe_router(_dev(h, "h", F32), K, _dev(w, "w"), _wf32(w, "w"), T, K, E, top,
+                                         _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), _stream()))
     return ids, wts
 
 
@@ -658,15 +679,17 @@ def sinkattn(proj: torch.Tensor, q_off: int, cache_k: torch.Tensor, cache_v: tor
 
 def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tensor, b_off: int, A_log: torch.Tensor,
                   dt_bias: torch.Tensor, *, H: int, G: int, d: int, per_channel: bool, q_scale: float,
-                  norm_eps: float = 1e-6):
+                  norm_eps: float = 1e-6, w_a2: Optional[torch.Tensor] = None):
     """qkv (T, 2 G d + H dv): q and k become unit vectors per head in place (q also times ``q_scale``). The raw decay
-    inputs are the H d (``per_channel``) or H columns of ``a`` at ``a_off``, the raw betas the H columns of ``b`` at
-    ``b_off``. Returns (dec, beta, kq): exp(-exp(A_log) softplus(a + dt_bias)) (T, H d) or (T, H), sigmoid(b) (T, H),
-    and k . q of the prepared vectors per key head (T, G)."""
+    inputs are the H d (``per_channel``) or H columns of ``a`` at ``a_off`` - or, with ``w_a2`` (H d or H, rank), w_a2
+    times the rank columns there; the raw betas are the H columns of ``b`` at ``b_off``. Returns (dec, beta, kq):
+    exp(-exp(A_log) softplus(a + dt_bias)) (T, H d) or (T, H), sigmoid(b) (T, H), and k . q of the prepared vectors
+    per key head (T, G)."""
     T, ld = qkv.shape
     n = H * d if per_channel else H
-    if a.shape[0] != T or b.shape[0] != T or a_off + n > a.shape[1] or b_off + H > b.shape[1] or \
-            A_log.numel() != H or dt_bias.numel() != n or ld < 2 * G * d:
+    cols = n if w_a2 is None else w_a2.shape[1]
+    if a.shape[0] != T or b.shape[0] != T or a_off + cols > a.shape[1] or b_off + H > b.shape[1] or \
+            A_log.numel() != H or dt_bias.numel() != n or ld < 2 * G * d or (w_a2 is not None and w_a2.shape[0] != n):
         raise ValueError("delta_prepare: shapes")
     dec = torch.empty(T, n, dtype=F32, device=qkv.device)
     beta = torch.empty(T, H, dtype=F32, device=qkv.device)
@@ -675,8 +698,40 @@ def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tenso
                                             _dev(b, "b", F32) + 4 * b_off, b.shape[1], _dev(A_log, "A_log", F32),
                                             _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), beta.data_ptr(),
                                             kq.data_ptr(), T, H, G, d, int(per_channel), float(q_scale),
-                                            float(norm_eps), _stream()))
+                                            float(norm_eps), _opt(w_a2, "w_a2"), 0 if w_a2 is None else w_a2.shape[1],
+                                            0 if w_a2 is None else _wf32(w_a2, "w_a2"), _stream()))
     return dec, beta, kq
+
+
+def delta_step_prepare(proj: torch.Tensor, off: int, conv_w: torch.Tensor, conv_state: torch.Tensor,
+                       seq_slot: torch.Tensor, seq_pos0: torch.Tensor, a_off: int, b_off: int, A_log: torch.Tensor,
+                       dt_bias: torch.Tensor, *, H: int, G: int, d: int, dv: int, per_channel: bool, q_scale: float,
+                       norm_eps: float = 1e-6, w_a2: Optional[torch.Tensor] = None):
+    """``conv_silu`` (without a bias) and ``delta_prepare`` in one launch for a step in which every sequence brings
+    one token: row b of ``proj`` belongs to sequence b; its q | k | v channels start at ``off``, the raw decay inputs
+    (or their rank inner values, with ``w_a2``) at ``a_off`` and the raw betas at ``b_off`` of the same row.
+    Returns (qkv (B, C), dec, beta, kq)."""
+    B, ld = proj.shape
+    C, taps = conv_w.shape
+    n = H * d if per_channel else H
+    cols = n if w_a2 is None else w_a2.shape[1]
+    if C != 2 * G * d + H * dv or off + C > ld or seq_slot.numel() != B or seq_pos0.numel() != B or \
+            tuple(conv_state.shape[1:]) != (max(1, taps - 1), C) or a_off + cols > ld or b_off + H > ld or \
+            A_log.numel() != H or dt_bias.numel() != n or (w_a2 is not None and w_a2.shape[0] != n):
+        raise ValueError("delta_step_prepare: shapes")
+    dev = proj.device
+    qkv = torch.empty(B, C, dtype=F32, device=dev)
+    dec = torch.empty(B, n, dtype=F32, device=dev)
+    beta = torch.empty(B, H, dtype=F32, device=dev)
+    kq = torch.empty(B, G, dtype=F32, device=dev)
+    base = _dev(proj, "proj", F32)
+    _check(load_library().lgs_delta_step_prepare(
+        base + 4 * off, ld, _dev(conv_w, "conv_w"), _wf32(conv_w, "conv_w"), taps, _dev(conv_state, "conv_state", F32),
+        _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32), qkv.data_ptr(), base + 4 * a_off, ld,
+        base + 4 * b_off, ld, _dev(A_log, "A_log", F32), _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), beta.data_ptr(),
+        kq.data_ptr(), B, H, G, d, dv, int(per_channel), float(q_scale), float(norm_eps), _opt(w_a2, "w_a2"),
+        0 if w_a2 is None else w_a2.shape[1], 0 if w_a2 is None else _wf32(w_a2, "w_a2"), _stream()))
+    return qkv, dec, beta, kq
 
 
 def gated_delta(qkv: torch.Tensor, dec: torch.Tensor, beta: torch.Tensor, kq: torch.Tensor, state: torch.Tensor,

@@ -447,6 +447,72 @@ def test_delta_prepare():
     assert (dec1.cpu().double() - w1).abs().max() < 1e-6
 
 
+@pytest.mark.parametrize("per_channel,taps", [(True, 4), (False, 1), (True, 2), (False, 7)])
+def test_one_token_step_form_equals_the_separate_launches(per_channel, taps):
+    """Convolution + preparation in one launch (with the low-rank second map inside) against conv_silu, the product
+    and delta_prepare, over steps that start one sequence over a stale history and continue two others; and the
+    low-rank gate inside the head gate against the product followed by the plain head gate."""
+    from lit_gpt import seq_ops
+    from lit_gpt.mixers import StepBatch
+
+    dev = torch.device("cuda", 0)
+    H, G, d, dv, rank = 4, 2, 6, 5, 3
+    C, n = 2 * G * d + H * dv, H * d if per_channel else H
+    g = torch.Generator().manual_seed(taps)
+    conv_w = torch.randn(C, taps, generator=g).to(dev)
+    w_a2 = torch.randn(n, rank, generator=g).to(dev) if per_channel else None
+    A_log, bias = torch.randn(H, generator=g).to(dev), torch.randn(n, generator=g).to(dev)
+    hist = max(1, taps - 1)
+    st_a = torch.randn(4, hist, C, generator=g).to(dev)
+    st_b = st_a.clone()
+    acols = rank if per_channel else H
+    ld = C + 3 + acols + H
+    pos = {0: 5, 2: 0, 3: 9}  # slot -> position: slot 2 starts a sequence over what the slot still holds
+    for it in range(3):
+        proj = torch.randn(3, ld, generator=g).to(dev)
+        step = StepBatch.build([(s, p, [0]) for s, p in pos.items()], dev)
+        kw = dict(H=H, G=G, d=d, per_channel=per_channel, q_scale=0.4)
+        qkv1, dec1, beta1, kq1 = seq_ops.delta_step_prepare(proj, 0, conv_w, st_a, step.seq_slot, step.seq_pos0, C + 3,
+                                                            C + 3 + acols, A_log, bias, dv=dv, w_a2=w_a2, **kw)
+        qkv2 = seq_ops.conv_silu(proj, 0, conv_w, torch.zeros(C, device=dev), st_b, step.seq_start, step.seq_slot,
+                                 step.seq_pos0, 1)
+        if per_channel:
+            a = torch.empty(3, n, device=dev)
+            seq_ops.linear(proj, w_a2, M=3, N=n, K=rank, y=a, a_off=C + 3, lda=ld, ldy=n)
+            dec2, beta2, kq2 = seq_ops.delta_prepare(qkv2, a, 0, proj, C + 3 + acols, A_log, bias, **kw)
+        else:
+            dec2, beta2, kq2 = seq_ops.delta_prepare(qkv2, proj, C + 3, proj, C + 3 + acols, A_log, bias, **kw)
+        for name, x, y in (("qkv", qkv1, qkv2), ("dec", dec1, dec2), ("beta", beta1, beta2), ("kq", kq1, kq2)):
+            assert (x - y).abs().max() < 1e-5, (it, name, (x - y).abs().max(1).values.tolist())
+        assert float((st_a - st_b).abs().max()) == 0.0, it
+        pos = {s: p + 1 for s, p in pos.items()}
+    o = torch.randn(3, H * dv, generator=g).to(dev)
+    w_g2 = torch.randn(H * dv, rank, generator=g).to(dev)
+    nw = torch.randn(dv, generator=g).to(dev)
+    gate = torch.empty(3, H * dv, device=dev)
+    seq_ops.linear(proj, w_g2, M=3, N=H * dv, K=rank, y=gate, a_off=2, lda=ld, ldy=H * dv)
+    kw = dict(H=H, dv=dv, unit_norm=True, eps=1e-5, act=seq_ops.ACT_SIGMOID, weight=nw, post=0.7)
+    want = seq_ops.head_gate(o.clone(), gate, 0, **kw)
+    got = seq_ops.head_gate(o.clone(), proj, 2, w_g2=w_g2, **kw)
+    assert (got - want).abs().max() < 1e-5
+
+
+def test_router_in_one_launch_equals_product_then_routing():
+    from lit_gpt import seq_ops
+
+    dev = torch.device("cuda", 0)
+    g = torch.Generator().manual_seed(8)
+    for E, K, top, dtype in ((5, 40, 3, torch.float32), (70, 33, 4, torch.float32), (18, 64, 4, torch.bfloat16)):
+        w = torch.randn(E, K, generator=g).to(dev, dtype)
+        h = torch.randn(6, K, generator=g).to(dev)
+        corr = (torch.randn(E, generator=g) * 0.05).to(dev)
+        z = torch.empty(6, E, device=dev)
+        seq_ops.linear(h, w, M=6, N=E, K=K, y=z, lda=K, ldy=E)
+        ids2, wts2 = seq_ops.moe_route_scores(z, 0, E, top, corr)
+        ids1, wts1 = seq_ops.moe_router(h, w, top, corr)
+        assert torch.equal(ids1, ids2) and (wts1 - wts2).abs().max() < 1e-5
+
+
 @pytest.mark.parametrize("schedule", ["whole", "portions", "single", "stale"])
 def test_state_carries_an_early_token(schedule):
     """With decay 1 (and beta one half) the memory keeps what the first tokens wrote for the whole sequence, so every
