@@ -198,6 +198,21 @@ def test_bf16_within_operand_noise():
     assert rel_err(whole, want).median() < TOL16 and rel_err(single, want).median() < TOL16
 
 
+@pytest.mark.parametrize("width,vocab", [(50, 300), (136, 70), (192, 97)])
+def test_bf16_without_routing_is_within_operand_noise_everywhere(width, vocab):
+    """No hard choices in the model: every row must be within bf16 operand noise, also at widths and head sizes that
+    are no multiples of the vector widths, as a whole prompt (MFMA tiles), in portions and token by token."""
+    layers = [(delta(heads=3, kv_heads=1, dim=10, vdim=14, conv=2), None),
+              (pair(heads=6, kv_heads=3, dim=6, vdim=10, every=7, rheads=2, rkv=2, rdim=20, rvdim=6), None),
+              (delta(heads=2, kv_heads=2, dim=16, vdim=24, conv=4), None)]
+    cfg = make_cfg(layers, width=width, vocab=vocab)
+    model, w = build(cfg, dtype=torch.bfloat16, seed=5)
+    toks = tokens_of(61, vocab, seed=3)
+    want = orc.forward(cfg, w, toks)
+    for cuts in ([61], [40] + [1] * 21, [13, 9, 20, 19]):
+        assert rel_err(engine_logits(model, [toks], [cuts])[0], want).max() < TOL16, cuts
+
+
 # ------------------------------------------------------------------------------------------------ schedules
 def slow_state(w):
     for k in w:
