@@ -335,6 +335,16 @@ class GatedDelta(InputReader):
 
     def forward(self, proj: torch.Tensor, step: StepBatch, cache: ScanState, x: torch.Tensor, accumulate: bool = True,
                 post: float = 1.0) -> None:
+        self.project(self.mix(proj, step, cache, post), x, accumulate)
+
+    def project(self, o: torch.Tensor, x: torch.Tensor, accumulate: bool) -> None:
+        """The out-projection of the gated head outputs ``o`` (T, H dv) into x (written or accumulated)."""
+        T, W = x.shape
+        seq_ops.linear(o, self.w_o, M=T, N=W, K=self.H * self.dv, y=x, lda=self.H * self.dv, ldy=W, accumulate=accumulate)
+
+    def mix(self, proj: torch.Tensor, step: StepBatch, cache: ScanState, post: float = 1.0) -> torch.Tensor:
+        """Everything before the out-projection: the gated, normed head outputs times ``post`` (T, H dv), fp32 or the
+        bf16 copy the out-projection's MFMA tiles read."""
         H, G, d, dv = self.H, self.G, self.d, self.dv
         T, ld = proj.shape
         tables = (step.seq_start, step.seq_slot, step.seq_pos0)
@@ -366,10 +376,8 @@ class GatedDelta(InputReader):
         o = seq_ops.gated_delta(qkv, dec, beta, kq, cache.s, *tables, H=H, G=G, d=d, dv=dv,
                                 per_channel=self.per_channel)
         act = seq_ops.ACT_SIGMOID if self.per_channel else seq_ops.ACT_SILU
-        o = seq_ops.head_gate(o, gate, g_off, H=H, dv=dv, unit_norm=True, eps=self.eps, act=act, weight=self.norm_w,
-                              post=post, bf16_copy=_tiles16(T, self.w_o), w_g2=g2)
-        W = x.shape[1]
-        seq_ops.linear(o, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
+        return seq_ops.head_gate(o, gate, g_off, H=H, dv=dv, unit_norm=True, eps=self.eps, act=act, weight=self.norm_w,
+                                 post=post, bf16_copy=_tiles16(T, self.w_o), w_g2=g2)
 
 
 class SinkAttention(InputReader):
@@ -417,7 +425,14 @@ class ParallelMixer(InputReader):
     """Two mixers side by side on the same input, summed with fixed factors: ``left_scale`` * a sink attention
     (tensors under ``left.``) + ``right_scale`` * a gated delta rule with one decay per head (``right.``). Both read
     the layer's one input projection; each factor is applied where its mixer's last elementwise kernel runs, and the
-    second out-projection accumulates onto the first."""
+    second out-projection accumulates onto the first. With ``overlap`` the delta rule's kernels of a prompt step run
+    on a second HIP stream (default priority) beside the attention's: they touch disjoint columns of the projection
+    and different caches; the second stream starts after the projection and is joined before the delta rule's
+    out-projection."""
+
+    overlap = True
+    OVERLAP_ROWS = 8  # steps of up to this many rows stay on one stream (a captured one-token step gains nothing)
+    _side: Dict[int, "torch.cuda.Stream"] = {}
 
     def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
         super().__init__()
@@ -439,8 +454,21 @@ class ParallelMixer(InputReader):
 
     def forward(self, proj: torch.Tensor, step: StepBatch, cache: CachePair, x: torch.Tensor,
                 accumulate: bool = True) -> None:
+        if not self.overlap or step.T <= self.OVERLAP_ROWS:
+            self.left(proj, step, cache.left, x, accumulate=accumulate, post=self.left_scale)
+            self.right(proj, step, cache.right, x, accumulate=True, post=self.right_scale)
+            return
+        main = torch.cuda.current_stream(proj.device)
+        index = proj.device.index or 0
+        side = self._side.get(index)
+        if side is None:
+            side = self._side[index] = torch.cuda.Stream(device=proj.device)
+        side.wait_stream(main)  # the projection is made
+        with torch.cuda.stream(side):
+            o = self.right.mix(proj, step, cache.right, post=self.right_scale)
         self.left(proj, step, cache.left, x, accumulate=accumulate, post=self.left_scale)
-        self.right(proj, step, cache.right, x, accumulate=True, post=self.right_scale)
+        main.wait_stream(side)
+        self.right.project(o, x, accumulate=True)
 
 
 class StreamLinks(nn.Module):

@@ -712,3 +712,23 @@ def test_checkpoint_folder_through_registry_and_runner(tmp_path):
     assert rel_err(got0, wa[[3, 9]]).max() < TOL32
     assert rel_err(got1, torch.stack([wa[10], wb[5]])).max() < TOL32
     assert rel_err(got3, wa[13:14]).max() < TOL32
+
+
+def test_two_streams_equal_one():
+    """The parallel mixer's branches on two streams against the same steps on one stream, bit for bit, over prompts,
+    portions and a batch (the second stream's kernels read only what was made before the fork)."""
+    from lit_gpt.mixers import ParallelMixer
+
+    cfg = make_cfg(MIXED)
+    model, _ = build(cfg, seed=13)
+    seqs = [tokens_of(n, cfg["vocab"], seed=20 + n) for n in (70, 33, 12)]
+    cuts = [[40, 30], [33], [0, 12]]
+    assert ParallelMixer.overlap
+    two = engine_logits(model, seqs, cuts, max_seq=80)
+    try:
+        ParallelMixer.overlap = False
+        one = engine_logits(model, seqs, cuts, max_seq=80)
+    finally:
+        ParallelMixer.overlap = True
+    for a, b in zip(one, two):
+        assert torch.equal(a, b)
