@@ -198,7 +198,7 @@ def test_bf16_within_operand_noise():
     assert rel_err(whole, want).median() < TOL16 and rel_err(single, want).median() < TOL16
 
 
-@pytest.mark.parametrize("width,vocab", [(50, 300), (136, 70), (192, 97)])
+@pytest.mark.parametrize("width,vocab", [(50, 300), (136, 70), (200, 97)])
 def test_bf16_without_routing_is_within_operand_noise_everywhere(width, vocab):
     """No hard choices in the model: every row must be within bf16 operand noise, also at widths and head sizes that
     are no multiples of the vector widths, as a whole prompt (MFMA tiles), in portions and token by token."""
