@@ -67,11 +67,12 @@ int lgs_gather_rows(const float* x, const int* rows, float* y, int n_rows, int W
  * workspace ws of B * max_chunks * H * d * dv floats (max_chunks = 64-token chunks of the longest sequence) the chunks
  * run side by side when sequences and heads alone would not fill the chip: local sums, a short carry over the
  * chunks, then the outputs. The prompt form rotates and scales q and k IN PLACE first (T_rows rows with positions
- * pos[T_rows]); the token-by-token form leaves them as they are. */
-int lgs_retention(float* q, float* k, const float* v, long ld, float* state, const float* decay,
+ * pos[T_rows]); the token-by-token form leaves them as they are. act (LGS_ACT_*): an activation on q, k and v as
+ * projected, ahead of the rotation and the scale (the prompt form applies it in place, to v as well). */
+int lgs_retention(float* q, float* k, float* v, long ld, float* state, const float* decay,
                   const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
                   int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked, float* ws, int max_chunks,
-                  int T_rows, const int* pos, lgs_stream_t stream);
+                  int T_rows, const int* pos, int act, lgs_stream_t stream);
 /* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * weight[i] * act(g[t * ldg + h * dv + i]) * post
  * (weight: dv values shared by the heads, or NULL). With w_g2 ([H dv][rank], bf16 or fp32 with g2_f32) g holds the
  * `rank` inner values of a low-rank gate per row and the gate's input is w_g2[h dv + i] . g[t * ldg ..]. */
@@ -107,12 +108,18 @@ int lgs_glu(const float* a, const float* b, long ld, void* out /* fp32, or bf16 
 int lgs_moe_route(const float* z, long ld, int T, int E, int top, int* ids, float* wts, lgs_stream_t stream);
 /* per token: s = softmax(z[t * ld .. + E]) over all E outputs; ids = the top largest of s + bias (bias NULL: of s;
  * lowest index first among equals), wts = s at those places (not renormalised). E <= 256. */
+/* sigmoid != 0: s = sigmoid(z) of every output on its own instead of the softmax. square != 0: wts = s^2 (the weight
+ * of an expert whose INPUT is scaled by s when its activation is the square of relu). */
 int lgs_moe_route_scores(const float* z, long ld, int T, int E, int top, const float* bias, int* ids, float* wts,
-                         lgs_stream_t stream);
+                         int sigmoid, int square, lgs_stream_t stream);
+/* out[t][i] = act(a[t * ld + i]) * (gate ? sigmoid(gate[t * ldg]) : 1), i < n: the activation of an ungated unit whose
+ * up-projection is part of a fused product, with an optional gate of one number per row */
+int lgs_act_rows(const float* a, long ld, const float* gate, long ldg, void* out /* fp32, or bf16 with out_bf16 */,
+                 int out_bf16, int T, int n, int act, lgs_stream_t stream);
 /* the router product z = w h[t] (w [E][K], fp32 sums) and lgs_moe_route_scores' routing in one launch: the form of
  * steps with few tokens */
 int lgs_moe_router(const float* h, long ldh, const void* w, int w_f32, int T, int K, int E, int top, const float* bias,
-                   int* ids, float* wts, lgs_stream_t stream);
+                   int* ids, float* wts, int sigmoid, int square, lgs_stream_t stream);
 /* streaming experts: actbuf[t * top + k] = act(up[ids[t][k]] h[t]), or with gated (up holds per expert F gate rows,
  * then F up rows) act(gate h) * (up h); x[t] (+)= sum_k wts[t][k] down[ids[t][k]] actbuf[..]. An id >= n_real names
  * an identity expert without matrices: it is skipped by lgs_moe_up and contributes wts * hin[t] in lgs_moe_down. */
@@ -165,33 +172,39 @@ int lgs_diffattn(const float* q, long ld, const void* cache_k, const void* cache
                  int max_len, int H, int G, int d, int dv, int max_seq, int chunk, float scale, float cap, float lambda,
                  float eps, float post, lgs_stream_t stream);
 
-/* ---- softmax attention with unit-RMS queries and keys and a sink ---- */
-/* Per token: every query head at proj[q_off ..] is divided by its root mean square (eps inside the root) and
- * multiplied by the query temperature 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: 1),
- * in place; every key head at proj[k_off ..] is divided by its root mean square on its way to cache_k
- * [slots][max_seq][G][d]; the values at proj[v_off ..] go to cache_v [slots][max_seq][G][dv] (bf16, or fp32). */
+/* ---- softmax attention with one map per head: normed and / or rotated queries and keys, a sink, a head gate ---- */
+/* Per token: every query head at proj[q_off ..] is (norm != 0) divided by its root mean square (eps inside the root)
+ * and multiplied by q_w [d] (NULL: no weight), then rotated on the pairs (i, i + rot_dims / 2) by position *
+ * inv_freq[i] (rot_dims 0: not), then multiplied by the query temperature
+ * 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: 1), in place; every key head at
+ * proj[k_off ..] is normed (k_w) and rotated alike on its way to cache_k [slots][max_seq][G][d], the projection
+ * itself stays as it is; the values at proj[v_off ..] go to cache_v [slots][max_seq][G][dv] (bf16, or fp32);
+ * v_off == k_off with dv == d makes the values the keys as projected. */
 int lgs_normattn_prepare(float* proj, long ld, int q_off, int k_off, int v_off, void* cache_k, void* cache_v,
                          int cache_f32, const int* slot, const int* pos, int T, int H, int G, int d, int dv, int max_seq,
-                         float eps, float temp_coef, int temp_every, lgs_stream_t stream);
+                         float eps, float temp_coef, int temp_every, int norm, const float* q_w, const float* k_w,
+                         const float* inv_freq, int rot_dims, lgs_stream_t stream);
 /* out[t][h] = post * sum_j p_j v_j over the cached rows j of the mask (as lgs_diffattn's), p = softmax of
  * cap((q . k_j) * scale) with exp(sink[h]) added to the normaliser (sink NULL: none); grouped key / value heads.
  * One map per head: q rows hold d values per head. max_len, splits and part (T H splits (2 + dv) floats) as in
- * lgs_diffattn. */
+ * lgs_diffattn. gate (NULL: none): head h's output at row t is multiplied by sigmoid(gate[t * ldg + h]). */
 int lgs_sinkattn(const float* q, long ld, const void* cache_k, const void* cache_v, int cache_f32, const float* sink,
                  const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, void* out_bf16, float* part,
                  int splits, int B, int max_len, int H, int G, int d, int dv, int max_seq, int chunk, float scale,
-                 float cap, float post, lgs_stream_t stream);
+                 float cap, float post, const float* gate, long ldg, lgs_stream_t stream);
 
 /* ---- gated delta rule ---- */
 /* Per token, on rows qkv [T][ld] = q [G][d] | k [G][d] | v [H][dv] (after their convolution): q and k become unit
  * vectors per head, x / sqrt(sum(x^2) + norm_eps), q also times q_scale, in place; beta[t][h] = sigmoid(b[t ldb + h]);
  * dec = exp(-exp(A_log[h]) softplus(a + dt_bias)) with a, dt_bias and dec per head and key channel ([H][d],
- * per_channel) or per head ([H]); kq[t][g] = k . q of the prepared vectors of key head g. */
+ * per_channel) or per head ([H]); kq[t][g] = k . q of the prepared vectors of key head g.
+ * unit 0: k stays as projected and q is only multiplied by q_scale. decay_form 1: dec = sigmoid(a + dt_bias)^(1 / tau)
+ * (A_log unused). b NULL: no betas (the plain rule of lgs_gated_delta). */
 int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb, const float* A_log,
                       const float* dt_bias, float* dec, float* beta, float* kq, int T, int H, int G, int d,
                       int per_channel, float q_scale, float norm_eps,
                       const void* w_a2 /* optional: a holds `rank` values per row, the raw input of entry i is w_a2[i] . a */,
-                      int rank, int a2_f32, lgs_stream_t stream);
+                      int rank, int a2_f32, int unit, int decay_form, float tau, lgs_stream_t stream);
 /* The same for a step in which every sequence brings ONE token (row b of u belongs to sequence b), with the short
  * causal convolution + silu of the C = 2 G d + H dv channels of u in the same launch: conv_w [C][taps] (column
  * taps - 1 weights the token itself, no bias), conv_state [slots][taps - 1][C] as in lgs_conv_silu (read unless the
@@ -204,10 +217,11 @@ int lgs_delta_step_prepare(const float* u, long ldu, const void* conv_w, int con
 /* Per sequence and head, token by token: S <- diag(dec) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q
  * (evaluated as S'^T q + u kq on the decayed state S', kq [T][G] = k . q from lgs_delta_prepare).
  * Head h reads q / k head h / (H / G). state [slots][H][d][dv] fp32 is read unless the sequence starts at position 0
- * and written back. d <= 512. lanes: lanes that share a state column (4, 8 or 16; 0: chosen from the sizes). */
+ * and written back. d <= 512. lanes: lanes that share a state column (4, 8 or 16; 0: chosen from the sizes).
+ * plain != 0: the gated rule without the correction, S <- diag(dec) S + k v^T, out = S^T q (beta unused). */
 int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, const float* kq, float* state,
                     const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, int B, int H, int G, int d,
-                    int dv, int per_channel, int lanes, lgs_stream_t stream);
+                    int dv, int per_channel, int lanes, int plain, lgs_stream_t stream);
 
 /* ---- selective state-space mixer ---- */
 /* out[t][c] = silu(bias[c] + sum_j w[c][j] u[t - (taps - 1 - j)][c]) per sequence of a packed batch; inputs before
@@ -233,6 +247,15 @@ int lgs_gated_group_norm(const float* y, const float* z, long ldz, const float* 
  * (limit <= 0: no clamps) */
 int lgs_glu_clamped(const float* a, const float* b, long ld, void* out, int out_bf16, int T, int n, float alpha,
                     float limit, float shift, lgs_stream_t stream);
+
+/* ---- sandwich norms ---- */
+/* One boundary between two sublayers whose input AND output are normed, rows of n values. With y0 (the sublayer that
+ * ran; y1: an optional second branch): b_i = w_i ? y_i / rms(y_i) * w_i : y_i, s = coef * (b_0 + b_1),
+ * x += s / rms(s) * post_w (post_w: the output norm's weight times the layer's per-channel scale). Then with next_w:
+ * h = x / rms(x) * next_w, the next sublayer's input, as fp32 (h) and / or rounded to bf16 (h_bf16). */
+int lgs_sandwich_step(float* x, const float* y0, const float* w0, const float* y1, const float* w1, float coef,
+                      const float* post_w, const float* next_w, float* h, void* h_bf16, float eps, int rows, int n,
+                      lgs_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -10,9 +10,10 @@
 //   lgs_diffattn_prepare  per token: rotary (interleaved pairs 2i, 2i + 1 of the first rot_dims dims of every map)
 //                         on the queries in place and on the keys on their way into the cache; values into the cache.
 //                         Without key / value columns (a layer that reads another layer's cache) only the queries.
-//   lgs_normattn_prepare  per token: queries divided by their root mean square and multiplied by a temperature that
-//                         grows with the position, in place; keys divided by their root mean square on their way
-//                         into the cache; values into the cache. No rotation.
+//   lgs_normattn_prepare  per token: queries optionally divided by their root mean square (optionally weighted),
+//                         optionally rotated (pairs i, i + rot_dims / 2) and multiplied by a temperature that grows
+//                         with the position, in place; keys normed and rotated alike on their way into the cache;
+//                         values (own columns, or the keys as projected) into the cache.
 //   lgs_diffattn,         QT consecutive queries of one sequence and one head per workgroup (8 with two maps, 16 with
 //   lgs_sinkattn          one) against key tiles of 256 cached rows: a thread per key for the scores, an online
 //                         softmax per (query, map), a thread per value column for the weighted sums. One query per
@@ -89,31 +90,61 @@ struct NormPrepArgs {
   const int *slot, *pos;
   int H, G, d, dv, S, temp_every;
   float eps, temp_coef;
+  int norm;                // 0: q and k as projected; 1: divided by their root mean square
+  const float *q_w, *k_w;  // optional weights [d] of the two norms, shared by the heads
+  const float* inv_freq;   // [rot_dims / 2]: rotary positions on pairs (i, i + rot_dims / 2) after the norm
+  int rot_dims;
 };
 
-// grid (T): wave w takes the vectors w, w + 4, ... of the H query heads (divided by their root mean square and
-// multiplied by the position's query temperature, in place) and of the G key heads (divided by their root mean
-// square on their way into the cache); then all threads copy the values into the cache.
+// grid (T): wave w takes the vectors w, w + 4, ... of the H query heads (normed, rotated and multiplied by the
+// position's query temperature, in place) and of the G key heads (normed and rotated on their way into the cache);
+// then all threads copy the values into the cache. The value columns may be the key columns themselves (values = the
+// keys as projected): the keys are never changed in place.
 template <bool CF32>
 __global__ void __launch_bounds__(256) normattn_prepare_kernel(NormPrepArgs p) {
   const size_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pos = p.pos[t], d = p.d;
+  const int pos = p.pos[t], d = p.d, half = p.rot_dims / 2;
+  if (pos < 0 || pos >= p.S) return;  // the host sizes the cache; never write out of bounds
   float* row = p.proj + t * p.ld;
   const size_t crow = ((size_t)p.slot[t] * p.S + pos) * p.G;
   const float temp = p.temp_every > 0 ? 1.0f + p.temp_coef * logf((float)((pos + 1) / p.temp_every + 1)) : 1.0f;
+  const float fpos = (float)pos;
   for (int vec = wave; vec < p.H + p.G; vec += 4) {
     const bool isk = vec >= p.H;
     float* x = row + (isk ? p.k_off + (size_t)(vec - p.H) * d : p.q_off + (size_t)vec * d);
-    float ss = 0.0f;
-    for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
-    ss = wave_sum(ss);
-    const float s = (isk ? 1.0f : temp) / sqrtf(ss / (float)d + p.eps);
-    for (int i = lane; i < d; i += 64) {
-      if (isk) cstore<CF32>(p.cache_k, (crow + (vec - p.H)) * d + i, x[i] * s);
-      else x[i] *= s;
+    const float* w = isk ? p.k_w : p.q_w;
+    float s = 1.0f;
+    if (p.norm) {
+      float ss = 0.0f;
+      for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
+      ss = wave_sum(ss);
+      s = 1.0f / sqrtf(ss / (float)d + p.eps);
+    }
+    const float post = isk ? 1.0f : temp;
+    const size_t kat = (crow + (vec - p.H)) * d;
+    for (int i = lane; i < half; i += 64) {  // a lane owns both members of a rotated pair
+      float u = x[i] * s, v = x[i + half] * s;
+      if (w) u *= w[i], v *= w[i + half];
+      float sn, cs;
+      sincosf(fpos * p.inv_freq[i], &sn, &cs);
+      const float a = (u * cs - v * sn) * post, b = (v * cs + u * sn) * post;
+      if (isk) {
+        cstore<CF32>(p.cache_k, kat + i, a);
+        cstore<CF32>(p.cache_k, kat + i + half, b);
+      } else {
+        x[i] = a;
+        x[i + half] = b;
+      }
+    }
+    for (int i = p.rot_dims + lane; i < d; i += 64) {
+      float u = x[i] * s;
+      if (w) u *= w[i];
+      if (isk) cstore<CF32>(p.cache_k, kat + i, u);
+      else x[i] = u * post;
     }
   }
+  __syncthreads();
   const int nv = p.G * p.dv;
   for (int i = threadIdx.x; i < nv; i += 256) cstore<CF32>(p.cache_v, crow * p.dv + i, row[p.v_off + i]);
 }
@@ -130,6 +161,8 @@ struct AttnArgs {
   int H, G, d, dv, S, chunk, tiles;
   float scale, cap, lambda, eps, post;
   const float* sink;  // one map: exp(sink[h]) joins the softmax normaliser (NULL: no sink)
+  const float* gate;  // one map: the head's output is multiplied by sigmoid(gate[row * ldg + h]) (NULL: not)
+  long ldg;
 };
 
 constexpr int kKeyTile = 256;
@@ -164,7 +197,8 @@ __device__ __forceinline__ void sink_finish(float a, float m, float l, const Att
     num = a * w;
   }
   if (c < p.dv) {
-    const float v = num / den * p.post;
+    float v = num / den * p.post;
+    if (p.gate) v *= sigmoid_f(p.gate[row * p.ldg + h]);
     const size_t at = row * p.H * p.dv + (size_t)h * p.dv + c;
     p.out[at] = v;
     if (p.out16) p.out16[at] = f2bf(v);
@@ -451,7 +485,7 @@ extern "C" int lgs_diffattn(const float* q, long ld, const void* cache_k, const 
   LGA_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || (part && max_len == 1)),
                 "lgs_diffattn: splits need one token per sequence and a workspace");
   lgs::AttnArgs p{q, ld, cache_k, cache_v, seq_start, seq_slot, seq_pos0, out, (uint16_t*)out_bf16, part,
-                  H, G, d, dv, max_seq, chunk, 0, scale, cap, lambda, eps, post, nullptr};
+                  H, G, d, dv, max_seq, chunk, 0, scale, cap, lambda, eps, post, nullptr, nullptr, 0};
   int rc;
   if (max_len == 1) {
     p.tiles = 1;
@@ -468,14 +502,18 @@ extern "C" int lgs_diffattn(const float* q, long ld, const void* cache_k, const 
 
 extern "C" int lgs_normattn_prepare(float* proj, long ld, int q_off, int k_off, int v_off, void* cache_k, void* cache_v,
                                     int cache_f32, const int* slot, const int* pos, int T, int H, int G, int d, int dv,
-                                    int max_seq, float eps, float temp_coef, int temp_every, hipStream_t stream) {
+                                    int max_seq, float eps, float temp_coef, int temp_every, int norm, const float* q_w,
+                                    const float* k_w, const float* inv_freq, int rot_dims, hipStream_t stream) {
   LGA_CHECK_ARG(proj && slot && pos && cache_k && cache_v && T > 0 && max_seq > 0, "lgs_normattn_prepare: bad arguments");
   LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && temp_every >= 0,
                 "lgs_normattn_prepare: heads must be a multiple of the key heads");
   LGA_CHECK_ARG(q_off >= 0 && q_off + (long)H * d <= ld && k_off >= 0 && k_off + (long)G * d <= ld && v_off >= 0 &&
                     v_off + (long)G * dv <= ld,
                 "lgs_normattn_prepare: queries, keys or values outside the row");
-  lgs::NormPrepArgs p{proj, ld, q_off, k_off, v_off, cache_k, cache_v, slot, pos, H, G, d, dv, max_seq, temp_every, eps, temp_coef};
+  LGA_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || inv_freq),
+                "lgs_normattn_prepare: rotary dims");
+  lgs::NormPrepArgs p{proj, ld, q_off, k_off, v_off, cache_k, cache_v, slot, pos, H, G, d, dv, max_seq, temp_every, eps,
+                      temp_coef, norm ? 1 : 0, q_w, k_w, inv_freq, rot_dims};
   if (cache_f32) lgs::normattn_prepare_kernel<true><<<T, 256, 0, stream>>>(p);
   else lgs::normattn_prepare_kernel<false><<<T, 256, 0, stream>>>(p);
   LGA_LAUNCH_RETURN();
@@ -484,15 +522,17 @@ extern "C" int lgs_normattn_prepare(float* proj, long ld, int q_off, int k_off, 
 extern "C" int lgs_sinkattn(const float* q, long ld, const void* cache_k, const void* cache_v, int cache_f32,
                             const float* sink, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
                             void* out_bf16, float* part, int splits, int B, int max_len, int H, int G, int d, int dv,
-                            int max_seq, int chunk, float scale, float cap, float post, hipStream_t stream) {
+                            int max_seq, int chunk, float scale, float cap, float post, const float* gate, long ldg,
+                            hipStream_t stream) {
   LGA_CHECK_ARG(q && cache_k && cache_v && seq_start && seq_slot && seq_pos0 && out, "lgs_sinkattn: null pointer");
+  LGA_CHECK_ARG(!gate || ldg >= H, "lgs_sinkattn: the head gates' row stride");
   LGA_CHECK_ARG(B > 0 && max_len > 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0, "lgs_sinkattn: bad sizes");
   LGA_CHECK_ARG(d > 0 && d <= 512 && dv > 0 && dv <= 256, "lgs_sinkattn: key dim <= 512, value dim <= 256");
   LGA_CHECK_ARG(ld >= (long)H * d && chunk >= 0 && max_seq > 0, "lgs_sinkattn: bad sizes");
   LGA_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || (part && max_len == 1)),
                 "lgs_sinkattn: splits need one token per sequence and a workspace");
   lgs::AttnArgs p{q, ld, cache_k, cache_v, seq_start, seq_slot, seq_pos0, out, (uint16_t*)out_bf16, part,
-                  H, G, d, dv, max_seq, chunk, 0, scale, cap, 0.0f, 0.0f, post, sink};
+                  H, G, d, dv, max_seq, chunk, 0, scale, cap, 0.0f, 0.0f, post, sink, gate, ldg};
   int rc;
   if (max_len == 1) {
     p.tiles = 1;

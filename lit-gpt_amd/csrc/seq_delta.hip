@@ -37,6 +37,10 @@ struct DeltaPrepArgs {
   // w_a2[i] . a (w_a2 [H d or H][rank], bf16 or fp32)
   const void* w_a2;
   int rank, a2_f32;
+  // unit: q and k become unit vectors (0: q is only scaled, k stays as it is). decay_form 0:
+  // exp(-exp(A_log) softplus(raw + dt_bias)); 1: sigmoid(raw + dt_bias)^(1 / tau) (A_log unused). b NULL: no betas.
+  int unit, decay_form;
+  float tau;
   // the fused one-token form only: the convolution's inputs u [B][ldu] (C = 2 G d + H dv channels), its weights
   // [C][taps] and its slot-indexed history [slots][taps - 1][C]
   const float* u;
@@ -46,6 +50,13 @@ struct DeltaPrepArgs {
   float* conv_state;
   const int *seq_slot, *seq_pos0;
 };
+
+// the decay of one entry from its raw input z (bias added): form 0 exp(-exp(A_log[head]) softplus(z)); form 1
+// sigmoid(z)^(1 / tau) = exp(-softplus(-z) / tau)
+__device__ __forceinline__ float decay_of(const DeltaPrepArgs& p, float z, int head) {
+  if (p.decay_form == 1) return expf(-softplus_d(-z) / p.tau);
+  return expf(-expf(p.A_log[head]) * softplus_d(z));
+}
 
 // One row's preparation by a whole workgroup: wave w makes the vectors w, w + 4, ... of the 2 G query / key heads
 // unit vectors; all threads walk the decays and betas; then k . q per key head.
@@ -65,16 +76,17 @@ __device__ __forceinline__ void delta_prepare_row(const DeltaPrepArgs& p, size_t
     float ss = 0.0f;
     for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
     ss = wave_sum(ss);
-    const float s = (vec < p.G ? p.q_scale : 1.0f) / sqrtf(ss + p.norm_eps);
-    for (int i = lane; i < d; i += 64) x[i] *= s;
+    const float s = p.unit ? (vec < p.G ? p.q_scale : 1.0f) / sqrtf(ss + p.norm_eps) : (vec < p.G ? p.q_scale : 1.0f);
+    if (s != 1.0f)
+      for (int i = lane; i < d; i += 64) x[i] *= s;
   }
   const int dc = p.per_channel ? d : 1, n = p.H * dc;
   for (int i = threadIdx.x; i < n; i += 256) {
-    const float rate = expf(p.A_log[i / dc]);
     const float raw = p.w_a2 ? lowrank_dot<A2F32>(p.w_a2, i, a1, p.rank) : p.a[t * p.lda + i];
-    p.dec[t * n + i] = expf(-rate * softplus_d(raw + p.dt_bias[i]));
+    p.dec[t * n + i] = decay_of(p, raw + p.dt_bias[i], i / dc);
   }
-  for (int h = threadIdx.x; h < p.H; h += 256) p.beta[t * p.H + h] = sigmoid_f(p.b[t * p.ldb + h]);
+  if (p.b)
+    for (int h = threadIdx.x; h < p.H; h += 256) p.beta[t * p.H + h] = sigmoid_f(p.b[t * p.ldb + h]);
   __syncthreads();  // the unit vectors of all heads are written
   for (int g = wave; g < p.G; g += 4) {
     const float *q = row + (size_t)g * d, *k = row + (size_t)(p.G + g) * d;
@@ -157,9 +169,8 @@ __global__ void __launch_bounds__(256) delta_step_prepare_kernel(DeltaPrepArgs p
     }
     const int i = blk * 256 + tid;
     if (i < n) {
-      const float rate = expf(p.A_log[i / dc]);
       const float raw = p.w_a2 ? lowrank_dot<A2F32>(p.w_a2, i, buf, p.rank) : p.a[(size_t)b * p.lda + i];
-      p.dec[(size_t)b * n + i] = expf(-rate * softplus_d(raw + p.dt_bias[i]));
+      p.dec[(size_t)b * n + i] = decay_of(p, raw + p.dt_bias[i], i / dc);
     }
     if (blk == 0)
       for (int h = tid; h < p.H; h += 256) p.beta[(size_t)b * p.H + h] = sigmoid_f(p.b[(size_t)b * p.ldb + h]);
@@ -178,6 +189,7 @@ struct DeltaArgs {
   int H, G, d, dv, per_channel;
   int ncb, items;  // column blocks per head; work items = B * H * ncb
 };
+// DELTA false: the plain gated rule S <- diag(g) S + k v^T (u = v: no correction towards the key's value, no beta)
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
@@ -203,7 +215,7 @@ __device__ __forceinline__ void lanes_sum2(float& a, float& b) {
 
 // grid (B * H * ceil(dv / CW) rounded up to 8), CW = 256 / LPC columns per workgroup. Lane l of a wave: r = l % LPC, column
 // l / LPC of the wave's 64 / LPC; the lane holds the rows 4 (r + LPC j) + e, j < NR4, e < 4, of its column.
-template <int NR4, int LPC>
+template <int NR4, int LPC, bool DELTA>
 __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
   constexpr int DP = 4 * NR4 * LPC;      // rows, padded
   constexpr int CW = 256 / LPC;          // columns per workgroup
@@ -257,13 +269,13 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
     } else if (e < 3 * DP + CW) {
       const int c = cblk * CW + (e - 3 * DP);
       if (c < dv) src[i] = p.qkv + (size_t)r0 * p.ld + (size_t)2 * p.G * d + (size_t)hd * dv + c, step[i] = p.ld;
-    } else if (e == 3 * DP + CW) {
+    } else if (e == 3 * DP + CW && DELTA) {
       src[i] = p.beta + (size_t)r0 * H + hd, step[i] = H;
     } else if (e == 3 * DP + CW + 1) {
       src[i] = p.kq + (size_t)r0 * p.G + g, step[i] = p.G;
     }
     has[i] = src[i] != nullptr;
-    if (!has[i]) src[i] = p.beta + (size_t)r0 * H + hd;
+    if (!has[i]) src[i] = p.kq + (size_t)r0 * p.G + g;
   }
   float pre[kDeltaTB][EPT];
   auto prefetch = [&](int t0) {
@@ -305,10 +317,12 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
         S[j][1] *= g4.y;
         S[j][2] *= g4.z;
         S[j][3] *= g4.w;
-        ka = fmaf(S[j][0], k4[j].x, ka);
-        kb = fmaf(S[j][1], k4[j].y, kb);
-        kc = fmaf(S[j][2], k4[j].z, kc);
-        kd = fmaf(S[j][3], k4[j].w, kd);
+        if (DELTA) {
+          ka = fmaf(S[j][0], k4[j].x, ka);
+          kb = fmaf(S[j][1], k4[j].y, kb);
+          kc = fmaf(S[j][2], k4[j].z, kc);
+          kd = fmaf(S[j][3], k4[j].w, kd);
+        }
         oa = fmaf(S[j][0], q4.x, oa);
         ob = fmaf(S[j][1], q4.y, ob);
         oc = fmaf(S[j][2], q4.z, oc);
@@ -316,7 +330,7 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
       }
       float ks = (ka + kb) + (kc + kd), qs = (oa + ob) + (oc + od);
       lanes_sum2<LPC>(ks, qs);
-      const float u = row[3 * DP + CW] * (row[3 * DP + cw] - ks);
+      const float u = DELTA ? row[3 * DP + CW] * (row[3 * DP + cw] - ks) : row[3 * DP + cw];
       if (r == 0) os[t][cw] = fmaf(u, row[3 * DP + CW + 1], qs);
 #pragma unroll
       for (int j = 0; j < NR4; ++j) {
@@ -344,16 +358,16 @@ __global__ void __launch_bounds__(256) gated_delta_kernel(DeltaArgs p) {
   }
 }
 
-template <int LPC>
+template <int LPC, bool DELTA>
 static bool gated_delta_launch(DeltaArgs p, int B, hipStream_t stream) {
   p.ncb = (p.dv + 256 / LPC - 1) / (256 / LPC);
   p.items = B * p.H * p.ncb;
   const dim3 grid((p.items + 7) / 8 * 8);
   const int nr4 = (p.d + 4 * LPC - 1) / (4 * LPC);
-  if (nr4 <= 1) gated_delta_kernel<1, LPC><<<grid, 256, 0, stream>>>(p);
-  else if (nr4 <= 2) gated_delta_kernel<2, LPC><<<grid, 256, 0, stream>>>(p);
-  else if (nr4 <= 4) gated_delta_kernel<4, LPC><<<grid, 256, 0, stream>>>(p);
-  else if (nr4 <= 8) gated_delta_kernel<8, LPC><<<grid, 256, 0, stream>>>(p);
+  if (nr4 <= 1) gated_delta_kernel<1, LPC, DELTA><<<grid, 256, 0, stream>>>(p);
+  else if (nr4 <= 2) gated_delta_kernel<2, LPC, DELTA><<<grid, 256, 0, stream>>>(p);
+  else if (nr4 <= 4) gated_delta_kernel<4, LPC, DELTA><<<grid, 256, 0, stream>>>(p);
+  else if (nr4 <= 8) gated_delta_kernel<8, LPC, DELTA><<<grid, 256, 0, stream>>>(p);
   else return false;
   return true;
 }
@@ -363,12 +377,15 @@ static bool gated_delta_launch(DeltaArgs p, int B, hipStream_t stream) {
 extern "C" int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, const float* b, long ldb,
                                  const float* A_log, const float* dt_bias, float* dec, float* beta, float* kq, int T,
                                  int H, int G, int d, int per_channel, float q_scale, float norm_eps, const void* w_a2,
-                                 int rank, int a2_f32, hipStream_t stream) {
-  LGA_CHECK_ARG(qkv && a && b && A_log && dt_bias && dec && beta && kq && T > 0, "lgs_delta_prepare: bad arguments");
+                                 int rank, int a2_f32, int unit, int decay_form, float tau, hipStream_t stream) {
+  LGA_CHECK_ARG(qkv && a && dt_bias && dec && kq && T > 0 && (!b || beta), "lgs_delta_prepare: bad arguments");
+  LGA_CHECK_ARG((decay_form == 0 && A_log) || (decay_form == 1 && tau > 0.0f),
+                "lgs_delta_prepare: decay form 0 needs A_log, form 1 a positive tau");
   LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && ld >= 2L * G * d, "lgs_delta_prepare: bad sizes");
   LGA_CHECK_ARG(!w_a2 || (rank > 0 && rank <= lgs::kMaxRank), "lgs_delta_prepare: inner size of the decay map 1..512");
   lgs::DeltaPrepArgs p{qkv, ld, a, lda, b, ldb, A_log, dt_bias, dec, beta, kq, H, G, d, per_channel ? 1 : 0, q_scale,
-                       norm_eps, w_a2, rank, a2_f32, nullptr, 0, nullptr, 0, 0, 0, nullptr, nullptr, nullptr};
+                       norm_eps, w_a2, rank, a2_f32, unit ? 1 : 0, decay_form, tau, nullptr, 0, nullptr, 0, 0, 0, nullptr,
+                       nullptr, nullptr};
   if (a2_f32) lgs::delta_prepare_kernel<true><<<T, 256, 0, stream>>>(p);
   else lgs::delta_prepare_kernel<false><<<T, 256, 0, stream>>>(p);
   LGA_LAUNCH_RETURN();
@@ -390,7 +407,8 @@ extern "C" int lgs_delta_step_prepare(const float* u, long ldu, const void* conv
   const int C = 2 * G * d + H * dv;
   LGA_CHECK_ARG(ldu >= C, "lgs_delta_step_prepare: channels outside the row");
   lgs::DeltaPrepArgs p{qkv, C, a, lda, b, ldb, A_log, dt_bias, dec, beta, kq, H, G, d, per_channel ? 1 : 0, q_scale,
-                       norm_eps, w_a2, rank, a2_f32, u, ldu, conv_w, conv_f32, taps, C, conv_state, seq_slot, seq_pos0};
+                       norm_eps, w_a2, rank, a2_f32, 1, 0, 1.0f, u, ldu, conv_w, conv_f32, taps, C, conv_state, seq_slot,
+                       seq_pos0};
   const int n = per_channel ? H * d : H;
   const dim3 grid(B, G + (H * dv + 255) / 256 + (n + 255) / 256);
   LGA_CHECK_ARG(d <= 512 && grid.y <= 65535, "lgs_delta_step_prepare: key dim <= 512");
@@ -406,8 +424,9 @@ extern "C" int lgs_delta_step_prepare(const float* u, long ldu, const void* conv
 
 extern "C" int lgs_gated_delta(const float* qkv, long ld, const float* dec, const float* beta, const float* kq,
                                float* state, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
-                               int B, int H, int G, int d, int dv, int per_channel, int lanes, hipStream_t stream) {
-  LGA_CHECK_ARG(qkv && dec && beta && kq && state && seq_start && seq_slot && seq_pos0 && out,
+                               int B, int H, int G, int d, int dv, int per_channel, int lanes, int plain,
+                               hipStream_t stream) {
+  LGA_CHECK_ARG(qkv && dec && (beta || plain) && kq && state && seq_start && seq_slot && seq_pos0 && out,
                 "lgs_gated_delta: null pointer");
   LGA_CHECK_ARG(B > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && d <= 512 && dv > 0,
                 "lgs_gated_delta: bad sizes (key dim <= 512)");
@@ -425,9 +444,9 @@ extern "C" int lgs_gated_delta(const float* qkv, long ld, const float* dec, cons
   }
   while (lpc < 16 && d > 32 * lpc) lpc <<= 1;
   bool ok;
-  if (lpc == 4) ok = lgs::gated_delta_launch<4>(p, B, stream);
-  else if (lpc == 8) ok = lgs::gated_delta_launch<8>(p, B, stream);
-  else if (lpc == 16) ok = lgs::gated_delta_launch<16>(p, B, stream);
+  if (lpc == 4) ok = plain ? lgs::gated_delta_launch<4, false>(p, B, stream) : lgs::gated_delta_launch<4, true>(p, B, stream);
+  else if (lpc == 8) ok = plain ? lgs::gated_delta_launch<8, false>(p, B, stream) : lgs::gated_delta_launch<8, true>(p, B, stream);
+  else if (lpc == 16) ok = plain ? lgs::gated_delta_launch<16, false>(p, B, stream) : lgs::gated_delta_launch<16, true>(p, B, stream);
   else ok = false;
   LGA_CHECK_ARG(ok, "lgs_gated_delta: lanes per column must be 4, 8 or 16 and cover the key dim");
   LGA_LAUNCH_RETURN();

@@ -120,11 +120,13 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__
     for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= den;
 }
 
-// one wave: s = softmax(z) over all E outputs (z: the token's router logits, global or LDS); the `top` largest of
-// s + bias (lowest index first among equals) are chosen, and their weights are s itself: not renormalised, without
-// the bias
+// one wave: s = softmax(z) over all E outputs (z: the token's router logits, global or LDS), or with `sigmoid`
+// s = sigmoid(z) of every output on its own; the `top` largest of s + bias (lowest index first among equals) are
+// chosen, and their weights are s itself: not renormalised, without the bias; `square`: s^2 (the weight of an expert
+// whose INPUT is scaled by s when its activation is the square of relu: relu(s a)^2 = s^2 relu(a)^2 for s > 0)
 __device__ __forceinline__ void route_scores_wave(const float* z, int E, int top, const float* __restrict__ bias,
-                                                  int* __restrict__ ids, float* __restrict__ wts, int lane) {
+                                                  int* __restrict__ ids, float* __restrict__ wts, int lane,
+                                                  bool sigmoid = false, bool square = false) {
   float s[4], c[4], mx = -INFINITY;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
@@ -135,10 +137,11 @@ __device__ __forceinline__ void route_scores_wave(const float* z, int E, int top
   float den = 0.0f;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    s[e] = lane + 64 * e < E ? expf(s[e] - mx) : 0.0f;
+    if (sigmoid) s[e] = lane + 64 * e < E ? sigmoid_f(s[e]) : 0.0f;
+    else s[e] = lane + 64 * e < E ? expf(s[e] - mx) : 0.0f;
     den += s[e];
   }
-  den = wave_sum(den);
+  den = sigmoid ? 1.0f : wave_sum(den);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int i = lane + 64 * e;
@@ -169,7 +172,7 @@ __device__ __forceinline__ void route_scores_wave(const float* z, int E, int top
     }
     if (lane == 0) {
       ids[k] = bi;
-      wts[k] = bs;
+      wts[k] = square ? bs * bs : bs;
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -179,9 +182,24 @@ __device__ __forceinline__ void route_scores_wave(const float* z, int E, int top
 
 __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* __restrict__ z, long ld, int E, int top,
                                                               const float* __restrict__ bias, int* __restrict__ ids,
-                                                              float* __restrict__ wts) {
+                                                              float* __restrict__ wts, int sigmoid, int square) {
   const size_t t = blockIdx.x;
-  route_scores_wave(z + t * ld, E, top, bias, ids + t * top, wts + t * top, threadIdx.x);
+  route_scores_wave(z + t * ld, E, top, bias, ids + t * top, wts + t * top, threadIdx.x, sigmoid != 0, square != 0);
+}
+
+// grid (T, ceil(n / 256)): out[t][i] = act(a[t * ld + i]) * (gate ? sigmoid(gate[t * ldg]) : 1): the activation of an
+// ungated unit whose up-projection is part of a fused product, with an optional gate of one number per row
+__global__ void __launch_bounds__(256) act_rows_kernel(const float* __restrict__ a, long ld,
+                                                       const float* __restrict__ gate, long ldg,
+                                                       float* __restrict__ out, uint16_t* __restrict__ out16, int n,
+                                                       int act) {
+  const size_t t = blockIdx.x;
+  const int i = blockIdx.y * 256 + threadIdx.x;
+  if (i >= n) return;
+  float v = act_f(act, a[t * ld + i]);
+  if (gate) v *= sigmoid_f(gate[t * ldg]);
+  if (out16) out16[t * n + i] = f2bf(v);
+  else out[t * n + i] = v;
 }
 
 // grid (T), 1024 threads: the router's logits of one token (wave w takes outputs w, w + 16, ...; fp32 sums, the
@@ -190,7 +208,8 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* __res
 template <bool WF32>
 __global__ void __launch_bounds__(1024) moe_router_kernel(const float* __restrict__ h, long ldh, const void* __restrict__ w,
                                                           int K, int E, int top, const float* __restrict__ bias,
-                                                          int* __restrict__ ids, float* __restrict__ wts) {
+                                                          int* __restrict__ ids, float* __restrict__ wts, int sigmoid,
+                                                          int square) {
   __shared__ float z[256];
   const size_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -202,7 +221,7 @@ __global__ void __launch_bounds__(1024) moe_router_kernel(const float* __restric
     if (lane == 0) z[e] = a0;
   }
   __syncthreads();
-  if (wave == 0) route_scores_wave(z, E, top, bias, ids + t * top, wts + t * top, lane);
+  if (wave == 0) route_scores_wave(z, E, top, bias, ids + t * top, wts + t * top, lane, sigmoid != 0, square != 0);
 }
 
 // grid (ceil(F / 8), pairs): pair = token * top + choice; act[pair][f] = act(up_e[f] . h_token); GATED: an expert's
@@ -402,20 +421,29 @@ extern "C" int lgs_moe_route(const float* z, long ld, int T, int E, int top, int
 }
 
 extern "C" int lgs_moe_route_scores(const float* z, long ld, int T, int E, int top, const float* bias, int* ids,
-                                    float* wts, hipStream_t stream) {
+                                    float* wts, int sigmoid, int square, hipStream_t stream) {
   LGA_CHECK_ARG(z && ids && wts && T > 0, "lgs_moe_route_scores: bad arguments");
   LGA_CHECK_ARG(E > 0 && E <= 256 && top > 0 && top <= E,
                 "lgs_moe_route_scores: experts must be <= 256 and top <= experts");
-  lgs::moe_route_scores_kernel<<<T, 64, 0, stream>>>(z, ld, E, top, bias, ids, wts);
+  lgs::moe_route_scores_kernel<<<T, 64, 0, stream>>>(z, ld, E, top, bias, ids, wts, sigmoid, square);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_act_rows(const float* a, long ld, const float* gate, long ldg, void* out, int out_bf16, int T, int n,
+                            int act, hipStream_t stream) {
+  LGA_CHECK_ARG(a && out && T > 0 && n > 0 && ld >= n && act >= 0 && act <= lgs::kActSigmoid, "lgs_act_rows: bad arguments");
+  const dim3 grid(T, (n + 255) / 256);
+  lgs::act_rows_kernel<<<grid, 256, 0, stream>>>(a, ld, gate, ldg, out_bf16 ? nullptr : (float*)out,
+                                                 out_bf16 ? (uint16_t*)out : nullptr, n, act);
   LGA_LAUNCH_RETURN();
 }
 
 extern "C" int lgs_moe_router(const float* h, long ldh, const void* w, int w_f32, int T, int K, int E, int top,
-                              const float* bias, int* ids, float* wts, hipStream_t stream) {
+                              const float* bias, int* ids, float* wts, int sigmoid, int square, hipStream_t stream) {
   LGA_CHECK_ARG(h && w && ids && wts && T > 0 && K > 0 && ldh >= K, "lgs_moe_router: bad arguments");
   LGA_CHECK_ARG(E > 0 && E <= 256 && top > 0 && top <= E, "lgs_moe_router: experts must be <= 256 and top <= experts");
-  if (w_f32) lgs::moe_router_kernel<true><<<T, 1024, 0, stream>>>(h, ldh, w, K, E, top, bias, ids, wts);
-  else lgs::moe_router_kernel<false><<<T, 1024, 0, stream>>>(h, ldh, w, K, E, top, bias, ids, wts);
+  if (w_f32) lgs::moe_router_kernel<true><<<T, 1024, 0, stream>>>(h, ldh, w, K, E, top, bias, ids, wts, sigmoid, square);
+  else lgs::moe_router_kernel<false><<<T, 1024, 0, stream>>>(h, ldh, w, K, E, top, bias, ids, wts, sigmoid, square);
   LGA_LAUNCH_RETURN();
 }
 

@@ -31,6 +31,7 @@ struct RetArgs {
   float k_scale;
   float* ws;       // chunk-parallel prompt form: [B * max_chunks][H][d][dv] local sums, then chunk-start states
   int max_chunks;  // chunks of 64 tokens of the longest sequence
+  int act;         // activation on q, k and v as projected (ahead of the rotation and the key scale)
 };
 
 // grid (B, H, ceil(dv / 64)): a workgroup owns 64 columns of one head's state; wave w owns rows [w NR, (w + 1) NR)
@@ -57,24 +58,24 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(RetArgs p) {
     for (int tid = threadIdx.x; tid < d; tid += 256) {
       const float* qr = p.q + (size_t)t * p.ld + (size_t)h * d;
       const float* kr = p.k + (size_t)t * p.ld + (size_t)h * d;
-      float qo = qr[tid], ko = kr[tid];
+      float qo = act_f(p.act, qr[tid]), ko = act_f(p.act, kr[tid]);
       if (tid < p.rot_dims) {
         const int j = tid < half ? tid : tid - half;
         float sn, cs;
         sincosf(pos * p.inv_freq[j], &sn, &cs);
         if (tid < half) {
-          qo = qo * cs - qr[tid + half] * sn;
-          ko = ko * cs - kr[tid + half] * sn;
+          qo = qo * cs - act_f(p.act, qr[tid + half]) * sn;
+          ko = ko * cs - act_f(p.act, kr[tid + half]) * sn;
         } else {
-          qo = qo * cs + qr[tid - half] * sn;
-          ko = ko * cs + kr[tid - half] * sn;
+          qo = qo * cs + act_f(p.act, qr[tid - half]) * sn;
+          ko = ko * cs + act_f(p.act, kr[tid - half]) * sn;
         }
       }
       qs[tid] = qo;
       ks[tid] = ko * p.k_scale;
     }
     __syncthreads();
-    const float vt = live ? p.v[(size_t)t * p.ld + (size_t)h * dv + col] : 0.0f;
+    const float vt = live ? act_f(p.act, p.v[(size_t)t * p.ld + (size_t)h * dv + col]) : 0.0f;
     float o = 0.0f;
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
@@ -110,11 +111,13 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(RetArgs p) {
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kRC = 64, kVS = 80, kAS = 66;
 
-// grid (T, H): rotary on q and k in place (pairs i, i + rot_dims / 2) and the key scale, ahead of the chunk kernels
-__global__ void __launch_bounds__(64) retention_rope_kernel(float* __restrict__ q, float* __restrict__ k, long ld,
+// grid (T, H): the activation on q, k and v, rotary on q and k (pairs i, i + rot_dims / 2) and the key scale, all in
+// place, ahead of the chunk kernels
+__global__ void __launch_bounds__(64) retention_rope_kernel(float* __restrict__ q, float* __restrict__ k,
+                                                            float* __restrict__ v, long ld,
                                                             const float* __restrict__ inv_freq,
-                                                            const int* __restrict__ pos, int d, int rot_dims,
-                                                            float k_scale) {
+                                                            const int* __restrict__ pos, int d, int dv, int rot_dims,
+                                                            float k_scale, int act) {
   const int t = blockIdx.x, h = blockIdx.y, half = rot_dims / 2;
   float* qr = q + (size_t)t * ld + (size_t)h * d;
   float* kr = k + (size_t)t * ld + (size_t)h * d;
@@ -123,14 +126,20 @@ __global__ void __launch_bounds__(64) retention_rope_kernel(float* __restrict__ 
     if (i < half) {
       float sn, cs;
       sincosf(fpos * inv_freq[i], &sn, &cs);
-      const float qu = qr[i], qv = qr[i + half], ku = kr[i], kv = kr[i + half];
+      const float qu = act_f(act, qr[i]), qv = act_f(act, qr[i + half]);
+      const float ku = act_f(act, kr[i]), kv = act_f(act, kr[i + half]);
       qr[i] = qu * cs - qv * sn;
       qr[i + half] = qv * cs + qu * sn;
       kr[i] = (ku * cs - kv * sn) * k_scale;
       kr[i + half] = (kv * cs + ku * sn) * k_scale;
     } else if (i >= rot_dims) {
-      kr[i] *= k_scale;
+      if (act != kActNone) qr[i] = act_f(act, qr[i]);
+      kr[i] = act_f(act, kr[i]) * k_scale;
     }
+  }
+  if (act != kActNone) {
+    float* vr = v + (size_t)t * ld + (size_t)h * dv;
+    for (int i = threadIdx.x; i < dv; i += 64) vr[i] = act_f(act, vr[i]);
   }
 }
 
@@ -812,23 +821,26 @@ __global__ void __launch_bounds__(256) latent_combine_kernel(const float* __rest
 
 }  // namespace lgs
 
-extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float* state, const float* decay,
+extern "C" int lgs_retention(float* q, float* k, float* v, long ld, float* state, const float* decay,
                              const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0,
                              float* out, int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked,
-                             float* ws, int max_chunks, int T_rows, const int* pos, hipStream_t stream) {
+                             float* ws, int max_chunks, int T_rows, const int* pos, int act, hipStream_t stream) {
+  LGA_CHECK_ARG(act >= 0 && act <= lgs::kActSigmoid, "lgs_retention: unknown activation");
   LGA_CHECK_ARG(q && k && v && state && decay && seq_start && seq_slot && seq_pos0 && out, "lgs_retention: null pointer");
   LGA_CHECK_ARG(B > 0 && H > 0 && H <= 65535 && d > 0 && d <= 512 && dv > 0, "lgs_retention: head dim must be in [1, 512]");
   LGA_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || inv_freq),
                 "lgs_retention: bad rotary dims");
   LGA_CHECK_ARG(!ws || max_chunks > 0, "lgs_retention: a workspace needs the longest sequence's chunk count");
   lgs::RetArgs p{q, k, v, ld, state, decay, inv_freq, seq_start, seq_slot, seq_pos0, out, H, d, dv, rot_dims, k_scale,
-                 ws, max_chunks};
+                 ws, max_chunks, act};
   const dim3 grid(B, H, (dv + 63) / 64);
   if (chunked && d <= 128) {  // a prompt: chunks of 64 tokens as fp32 matrix products
     LGA_CHECK_ARG(T_rows > 0 && pos, "lgs_retention: the prompt form needs the row count and the rows' positions");
-    if (rot_dims > 0 || k_scale != 1.0f)
-      lgs::retention_rope_kernel<<<dim3(T_rows, H), 64, 0, stream>>>((float*)q, (float*)k, ld, inv_freq, pos, d, rot_dims,
-                                                                     k_scale);
+    if (rot_dims > 0 || k_scale != 1.0f || act != lgs::kActNone) {
+      lgs::retention_rope_kernel<<<dim3(T_rows, H), 64, 0, stream>>>(q, k, v, ld, inv_freq, pos, d, dv, rot_dims, k_scale,
+                                                                     act);
+      p.act = lgs::kActNone;  // applied in place: the chunk kernels read the activated values
+    }
     const size_t lds = lgs::retention_chunk_lds(d);
     const bool side = ws && (long)B * H * ((dv + 63) / 64) < lga::num_cu() && (long)B * max_chunks <= 1 << 24;
     const dim3 cgrid(side ? B * max_chunks : B, H, (dv + 63) / 64);

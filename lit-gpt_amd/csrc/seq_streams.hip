@@ -184,6 +184,97 @@ static bool streams_step_reg(const StreamArgs& p, int T, hipStream_t stream) {
   return true;
 }
 
+// ------------------------------------------------------------------------------------------------ sandwich norms
+// One boundary between two sublayers of a layer whose sublayers are normed on the way in AND on the way out.
+// With y0 (the sublayer that ran; up to two branches): b_i = w_i ? y_i / rms(y_i) * w_i : y_i, s = coef * sum_i b_i,
+// x <- x + s / rms(s) * post_w (post_w: the output norm's weight times the layer's per-channel scale). Then with
+// next_w: h = x / rms(x) * next_w, the next sublayer's input (fp32 and / or its bf16 rounding). Every root mean
+// square has eps inside the root. grid (rows); a row lives in registers up to 256 * CPT columns, else it is re-read.
+struct SandwichArgs {
+  float* x;
+  const float *y0, *w0, *y1, *w1;
+  float coef;
+  const float* post_w;
+  const float* next_w;
+  float* h;
+  uint16_t* h16;
+  float eps;
+  int n;
+};
+
+template <int CPT>
+__global__ void __launch_bounds__(256) sandwich_step_kernel(SandwichArgs p) {
+  __shared__ float red[4];
+  const size_t r = blockIdx.x;
+  const int n = p.n, tid = threadIdx.x;
+  float* xr = p.x + r * n;
+  const float inv_n = 1.0f / (float)n;
+  float xv[CPT];
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) xv[e] = tid + 256 * e < n ? xr[tid + 256 * e] : 0.0f;
+  if (p.y0) {
+    const float *a = p.y0 + r * n, *b = p.y1 ? p.y1 + r * n : nullptr;
+    float av[CPT], bv[CPT];
+    float sa = 0.0f, sb = 0.0f;
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) {
+      const int i = tid + 256 * e;
+      av[e] = i < n ? a[i] : 0.0f;
+      bv[e] = (b && i < n) ? b[i] : 0.0f;
+      sa = fmaf(av[e], av[e], sa);
+      sb = fmaf(bv[e], bv[e], sb);
+    }
+    for (int i = tid + 256 * CPT; i < n; i += 256) {
+      sa = fmaf(a[i], a[i], sa);
+      if (b) sb = fmaf(b[i], b[i], sb);
+    }
+    float ra = 1.0f, rb = 1.0f;
+    if (p.w0) ra = 1.0f / sqrtf(block_sum_256(sa, red) * inv_n + p.eps);
+    if (b && p.w1) rb = 1.0f / sqrtf(block_sum_256(sb, red) * inv_n + p.eps);
+    auto joined = [&](int i, float ya, float yb) {
+      float s = p.w0 ? ya * ra * p.w0[i] : ya;
+      if (b) s += p.w1 ? yb * rb * p.w1[i] : yb;
+      return s * p.coef;
+    };
+    float ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) {
+      const int i = tid + 256 * e;
+      av[e] = i < n ? joined(i, av[e], bv[e]) : 0.0f;  // (av now holds the joined value)
+      ss = fmaf(av[e], av[e], ss);
+    }
+    for (int i = tid + 256 * CPT; i < n; i += 256) {
+      const float s = joined(i, a[i], b ? b[i] : 0.0f);
+      ss = fmaf(s, s, ss);
+    }
+    const float rs = 1.0f / sqrtf(block_sum_256(ss, red) * inv_n + p.eps);
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) {
+      const int i = tid + 256 * e;
+      if (i < n) {
+        xv[e] = fmaf(av[e] * rs, p.post_w[i], xv[e]);
+        xr[i] = xv[e];
+      }
+    }
+    for (int i = tid + 256 * CPT; i < n; i += 256) xr[i] = fmaf(joined(i, a[i], b ? b[i] : 0.0f) * rs, p.post_w[i], xr[i]);
+  }
+  if (!p.next_w) return;
+  float sx = 0.0f;
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) sx = fmaf(xv[e], xv[e], sx);
+  for (int i = tid + 256 * CPT; i < n; i += 256) sx = fmaf(xr[i], xr[i], sx);  // (written by this thread above)
+  const float rx = 1.0f / sqrtf(block_sum_256(sx, red) * inv_n + p.eps);
+  auto put = [&](int i, float v) {
+    const float o = v * rx * p.next_w[i];
+    if (p.h) p.h[r * n + i] = o;
+    if (p.h16) p.h16[r * n + i] = f2bf(o);
+  };
+#pragma unroll
+  for (int e = 0; e < CPT; ++e)
+    if (tid + 256 * e < n) put(tid + 256 * e, xv[e]);
+  for (int i = tid + 256 * CPT; i < n; i += 256) put(i, xr[i]);
+}
+
 }  // namespace lgs
 
 extern "C" int lgs_embed_streams(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W,
@@ -211,5 +302,20 @@ extern "C" int lgs_streams_step(float* x, const float* y, const float* mix, cons
   else if (streams <= 4) done = lgs::streams_step_reg<4>(p, T, stream);
   else done = lgs::streams_step_reg<8>(p, T, stream);
   if (!done) lgs::streams_step_kernel<<<T, 256, 0, stream>>>(p);  // wide rows: column blocks one after the other
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_sandwich_step(float* x, const float* y0, const float* w0, const float* y1, const float* w1,
+                                 float coef, const float* post_w, const float* next_w, float* h, void* h_bf16, float eps,
+                                 int rows, int n, hipStream_t stream) {
+  LGA_CHECK_ARG(x && rows > 0 && n > 0, "lgs_sandwich_step: bad arguments");
+  LGA_CHECK_ARG(!y0 || post_w, "lgs_sandwich_step: a sublayer's output needs the output norm's weight");
+  LGA_CHECK_ARG(y0 || !y1, "lgs_sandwich_step: a second branch without a first");
+  LGA_CHECK_ARG(y0 || next_w, "lgs_sandwich_step: nothing to do");
+  LGA_CHECK_ARG(!next_w || h || h_bf16, "lgs_sandwich_step: the next input needs a place");
+  lgs::SandwichArgs p{x, y0, w0, y1, w1, coef, post_w, next_w, h, (uint16_t*)h_bf16, eps, n};
+  if (n <= 1024) lgs::sandwich_step_kernel<4><<<rows, 256, 0, stream>>>(p);
+  else if (n <= 2048) lgs::sandwich_step_kernel<8><<<rows, 256, 0, stream>>>(p);
+  else lgs::sandwich_step_kernel<16><<<rows, 256, 0, stream>>>(p);
   LGA_LAUNCH_RETURN();
 }

@@ -14,6 +14,7 @@ the tiny configs the test-suite uses.
 from __future__ import annotations
 
 import json
+import math
 from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Any, Dict, List, Literal, Optional, Type, Union
@@ -170,10 +171,25 @@ name_to_config: Dict[str, Dict[str, Any]] = {c["name"]: c for c in configs}
 class RotarySpec:
     dims: int = 0
     base: float = 10000.0
+    # band-wise rescaling of the frequencies for contexts longer than the ``original`` one: wavelengths above
+    # original / low are slowed down by ``factor``, those below original / high are kept, the band between blends
+    # the two linearly in original / wavelength. Keys: factor, low, high, original.
+    scaling: Optional[Dict[str, float]] = None
 
     def inv_freq(self) -> List[float]:
-        """f_i = base^(-2i / dims), i < dims / 2, in double precision (rounded once to fp32 by the caller)."""
-        return [float(self.base) ** (-2.0 * i / self.dims) for i in range(self.dims // 2)]
+        """f_i = base^(-2i / dims), i < dims / 2, rescaled band by band when ``scaling`` is set; in double precision
+        (rounded once to fp32 by the caller)."""
+        out = [float(self.base) ** (-2.0 * i / self.dims) for i in range(self.dims // 2)]
+        if self.scaling:
+            factor, low, high, orig = (float(self.scaling[k]) for k in ("factor", "low", "high", "original"))
+            for i, f in enumerate(out):
+                wavelength = 2.0 * math.pi / f
+                if wavelength > orig / low:
+                    out[i] = f / factor
+                elif wavelength >= orig / high:
+                    mix = (orig / wavelength - low) / (high - low)
+                    out[i] = (1.0 - mix) * f / factor + mix * f
+        return out
 
 
 @dataclass
@@ -204,6 +220,14 @@ class MixerSpec:
     right: Optional["MixerSpec"] = None
     left_scale: float = 1.0  # ... and are summed with these factors
     right_scale: float = 1.0
+    branch_norm: bool = False  # parallel: each branch's output is RMS-normed over the width (weights "left.out" /
+    # "right.out") before the weighted sum
+    # one-map softmax attention ("sink_attention" and its relatives):
+    qk_norm: str = "unit"  # "none" | "unit" (divided by the root mean square) | "weight" (and times "q.norm" / "k.norm")
+    sink_kind: str = "learned"  # "none" | "learned" (a scalar per head, "sink") | "one" (a sink of score 0: 1 + sum exp)
+    values: str = "own"  # "own" (a value projection) | "keys" (the keys as projected, before their norm)
+    head_gate: bool = False  # every head's output times sigmoid(W_g h)_h, one number per head ("g")
+    tau: float = 0.0  # gated_linear: the decay is sigmoid(z)^(1 / tau)
 
 
 @dataclass
@@ -214,6 +238,7 @@ class FeedForwardSpec:
     top: int = 0
     limit: float = 0.0  # clamped gated unit: bound of the gate (from above) and of the up branch (both sides)
     identity: int = 0  # moe: router outputs beyond ``experts`` that stand for identity experts (output = input)
+    shared_ff: int = 0  # moe: size of a shared expert that runs for every token behind a sigmoid gate (0: none)
 
 
 @dataclass
@@ -224,9 +249,14 @@ class LayerSpec:
 
 # "channel_delta" / "gated_delta": the gated delta rule with a decay per head and key channel / per head;
 # "sink_attention": softmax attention with unit-RMS queries and keys, a query temperature and a sink;
-# "parallel": a sink attention and a gated delta rule side by side
+# "rotary_attention": grouped softmax attention with rotary positions (half layout) and a sink of score 0;
+# "key_value_attention": softmax attention whose values are the keys as projected, weighted q / k norms, a query
+# temperature and a gate per head; "gated_linear": the gated rule without the correction and a decay per key channel,
+# S <- diag(alpha) S + k v^T; "lightning": the constant-decay rule on silu(q), silu(k), silu(v);
+# "parallel": two of these side by side (which two, the design says)
 MIXER_KINDS = ("retention", "latent_attention", "attention", "mamba2", "channel_delta", "gated_delta",
-               "sink_attention", "parallel")
+               "sink_attention", "parallel", "rotary_attention", "key_value_attention", "gated_linear", "lightning")
+SOFTMAX_KINDS = ("sink_attention", "rotary_attention", "key_value_attention")
 
 
 @dataclass(frozen=True)
@@ -235,22 +265,33 @@ class LayeredDesign:
 
     # "parallel": x += mixer(h) + ff(h), one norm; "sequential": x += mixer(norm1 x), then x += ff(norm2 x);
     # "post": the sublayers read x itself and their OUTPUT is normed: x += m norm1(mixer(x)), then x += m norm2(ff(x))
+    # "sandwich": normed on the way in and out, with a per-channel scale: x += ls1 * norm1b(mixer(norm1 x)), then
+    # x += ls2 * norm2b(ff(norm2 x))
     block: str
     norm_offset: float  # the norm multiplies by offset + stored weight
     tied_head: bool  # logits from the embedding table itself, or from a matrix of their own ("head")
-    dense_ff: str  # "gelu_tanh": W_down(gelu_tanh(gate) * up); "clamped_swish": g sigmoid(1.702 g) (u + 1), clamped
+    # "gelu_tanh": W_down(gelu_tanh(gate) * up); "clamped_swish": g sigmoid(1.702 g) (u + 1), clamped;
+    # "relu2": W_down relu(W_up h)^2 (no gate)
+    dense_ff: str
     norm: str = "rms"  # "rms": x / rms(x) * w; "layer": (x - mean) / sqrt(var + eps) * w + b (tensor "<norm>.b")
     positions: str = "none"  # "learned": a table "pos" whose row p joins the embedding at position p
     # "top_logits": the largest router logits, softmax over the chosen, experts W_down relu(W_up h)^2;
     # "scores": softmax over all router outputs (+ a stored correction for the choice only), weights = the chosen
     # scores as they are, gated experts W_down(silu(W_gate h) * W_up h), optional identity experts
+    # "sigmoid": scores = sigmoid of every router output, the largest chosen, the score scales the expert's INPUT,
+    # experts W_down relu(W_up h)^2, optional shared expert behind a sigmoid gate per token
     moe: str = "top_logits"
+    # layer type (config.json) -> (left kind, right kind, branch_norm) of the designs' two-branch mixers
+    pairs: Dict[str, tuple] = field(default_factory=lambda: {"parallel": ("sink_attention", "gated_delta", False)})
 
 
 DESIGNS: Dict[str, LayeredDesign] = {
     "Bavesun": LayeredDesign("parallel", 1.0, True, "gelu_tanh"),
     "Rigulorn": LayeredDesign("sequential", 0.0, False, "clamped_swish"),
     "Ravelorn": LayeredDesign("post", 0.0, False, "gelu_tanh", norm="layer", positions="learned", moe="scores"),
+    "Gatutar": LayeredDesign("sandwich", 0.0, False, "relu2", moe="sigmoid",
+                             pairs={"parallel": ("rotary_attention", "gated_linear", True),
+                                    "parallel_2": ("key_value_attention", "lightning", True)}),
 }
 
 
@@ -297,10 +338,25 @@ class LayeredConfig:
                 if not 0 < f.top <= f.experts + f.identity or f.identity < 0 or f.experts + f.identity > 256:
                     raise ValueError(f"layer {i}: top {f.top} of {f.experts} + {f.identity} experts (at most 256)")
             parts = [m.left, m.right] if m.kind == "parallel" else [m]
-            if m.kind == "parallel" and (m.left is None or m.left.kind != "sink_attention" or m.right is None or
-                                         m.right.kind != "gated_delta"):
-                raise ValueError(f"layer {i}: a parallel mixer holds a sink attention (left) and a gated delta rule (right)")
+            if m.kind == "parallel":
+                allowed = {(a, b) for a, b, _ in self.design.pairs.values()}
+                if m.left is None or m.right is None or (m.left.kind, m.right.kind) not in allowed:
+                    raise ValueError(f"layer {i}: a parallel mixer of this design holds one of {sorted(allowed)}")
             for q in parts:
+                if q.kind in ("gated_linear", "lightning"):
+                    if q.heads < 1 or not 1 <= q.dim <= 512 or q.vdim < 1:
+                        raise ValueError(f"layer {i}: heads {q.heads} / key dim {q.dim} (<= 512) / value dim {q.vdim}")
+                    if q.kind == "gated_linear" and not q.tau > 0.0:
+                        raise ValueError(f"layer {i}: tau must be positive")
+                    if q.kind == "lightning" and (q.decay is None or len(q.decay) != q.heads):
+                        raise ValueError(f"layer {i}: one decay per head")
+                if q.kind in ("rotary_attention", "key_value_attention"):
+                    if q.kv_heads < 1 or q.heads % q.kv_heads or not 1 <= q.dim <= 512 or not 1 <= q.vdim <= 256:
+                        raise ValueError(f"layer {i}: heads {q.heads} / key heads {q.kv_heads} / dims {q.dim}, {q.vdim}")
+                    if q.rot.dims % 2 or q.rot.dims > q.dim or q.q_temp_every < 0:
+                        raise ValueError(f"layer {i}: rotary dims {q.rot.dims} / q_temp.every {q.q_temp_every}")
+                    if q.values == "keys" and q.vdim != q.dim:
+                        raise ValueError(f"layer {i}: values that are the keys have the keys' size")
                 if q.kind in ("channel_delta", "gated_delta"):
                     if q.kv_heads < 1 or q.heads % q.kv_heads or not 1 <= q.dim <= 512 or q.vdim < 1:
                         raise ValueError(f"layer {i}: heads {q.heads} / key heads {q.kv_heads} / key dim {q.dim} (<= 512)")
@@ -311,7 +367,8 @@ class LayeredConfig:
                         raise ValueError(f"layer {i}: heads {q.heads} / key heads {q.kv_heads} / dims {q.dim}, {q.vdim}")
                     if q.q_temp_every < 0:
                         raise ValueError(f"layer {i}: q_temp.every must be positive")
-            if m.kind in ("channel_delta", "gated_delta", "sink_attention", "parallel"):
+            if m.kind in ("channel_delta", "gated_delta", "sink_attention", "parallel", "rotary_attention",
+                          "key_value_attention", "gated_linear", "lightning"):
                 continue
             if m.kind == "retention" and (m.decay is None or len(m.decay) != m.heads):
                 raise ValueError(f"layer {i}: retention needs one decay per head")
@@ -342,17 +399,29 @@ class LayeredConfig:
         return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, len(self.layers)))
 
     @staticmethod
-    def _mixer_spec(kind: str, m: Dict[str, Any]) -> MixerSpec:
-        if kind == "parallel":
-            return MixerSpec(kind=kind, heads=0, dim=0, vdim=0, rot=RotarySpec(),
-                             left=LayeredConfig._mixer_spec("sink_attention", m["left"]),
-                             right=LayeredConfig._mixer_spec("gated_delta", m["right"]),
-                             left_scale=float(m.get("left_scale", 1.0)), right_scale=float(m.get("right_scale", 1.0)))
+    def _mixer_spec(kind: str, m: Dict[str, Any], design: Optional[LayeredDesign] = None) -> MixerSpec:
+        pairs = (design or DESIGNS["Ravelorn"]).pairs
+        if kind in pairs:
+            left, right, normed = pairs[kind]
+            half = 0.5 if normed else 1.0  # normed branches are averaged
+            return MixerSpec(kind="parallel", heads=0, dim=0, vdim=0, rot=RotarySpec(),
+                             left=LayeredConfig._mixer_spec(left, m["left"]),
+                             right=LayeredConfig._mixer_spec(right, m["right"]),
+                             left_scale=float(m.get("left_scale", half)), right_scale=float(m.get("right_scale", half)),
+                             branch_norm=normed)
         rot = m.get("rot") or {}
         mask = m.get("mask") or {}
         temp = m.get("q_temp") or {}
+        extra = {}
+        if kind == "rotary_attention":
+            extra = dict(qk_norm="none", sink_kind="one")
+        elif kind == "key_value_attention":
+            extra = dict(qk_norm="weight", sink_kind="none", values="keys", head_gate=True)
+        scaling = rot.get("scaling")
         return MixerSpec(kind=kind, heads=int(m["heads"]), dim=int(m.get("dim", 0)), vdim=int(m["vdim"]),
-                         rot=RotarySpec(int(rot.get("dims", 0)), float(rot.get("base", 10000.0))),
+                         rot=RotarySpec(int(rot.get("dims", 0)), float(rot.get("base", 10000.0)),
+                                        {k: float(v) for k, v in scaling.items()} if scaling else None),
+                         tau=float(m.get("tau", 0.0)), **extra,
                          decay=[float(x) for x in m["decay"]] if "decay" in m else None,
                          kv_rank=int(m.get("kv_rank", 0)), rot_dim=int(m.get("rot_dim", 0)),
                          scale=float(m.get("scale", 1.0)), kv_heads=int(m.get("kv_heads", m["heads"])),
@@ -367,9 +436,10 @@ class LayeredConfig:
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "LayeredConfig":
         layers = []
+        design = DESIGNS.get(d["architecture"])
         for entry in d["layers"]:
             m = entry["mixer"]
-            mixer = cls._mixer_spec(entry["type"], m)
+            mixer = cls._mixer_spec(entry["type"], m, design)
             f = entry.get("mlp")
             if f is None:
                 mlp = None
@@ -377,7 +447,8 @@ class LayeredConfig:
                 mlp = FeedForwardSpec("dense", int(f["ff"]), limit=float(f.get("limit") or 0.0))
             elif f["kind"] == "moe":
                 mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]),
-                                      identity=int(f["router"].get("identity") or 0))
+                                      identity=int(f["router"].get("identity") or 0),
+                                      shared_ff=int((f.get("shared") or {}).get("ff") or 0))
             else:
                 raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
             layers.append(LayerSpec(mixer, mlp))
@@ -398,7 +469,8 @@ class LayeredConfig:
 
 
 # architecture name (config.json) -> "module:class" of the model that serves it
-ARCHITECTURES: Dict[str, str] = {name: "lit_gpt.layered:LayeredGPT" for name in ("Bavesun", "Rigulorn", "Ravelorn")}
+ARCHITECTURES: Dict[str, str] = {name: "lit_gpt.layered:LayeredGPT"
+                                 for name in ("Bavesun", "Rigulorn", "Ravelorn", "Gatutar")}
 
 
 def load_config(checkpoint_dir: Union[str, Path]) -> Union[Config, LayeredConfig]:

@@ -21,6 +21,11 @@ The design named by ``config.architecture`` fixes the layer's shape (``config.de
   and its output is written into all of them while a small matrix mixes them (``lit_gpt.mixers.StreamLinks``; one
   stream with unit weights is the plain residual sum). The write-back of a sublayer and the read + norm of the next
   run as one launch. Logits from a matrix of their own (``head``) after the final norm of the streams' sum.
+* sandwich — every sublayer is normed on the way in AND on the way out, and its normed output is scaled channel by
+  channel before it joins the residual: x <- x + ls1 * norm1b(mixer(norm1 x)), then x <- x + ls2 * norm2b(ff(norm2 x))
+  (RMS norms with plain weights). A two-branch mixer whose branches are each normed over the width hands both
+  outputs to the boundary launch, which norms and averages them, applies the output norm and the scale, adds the
+  residual and leaves the next sublayer's normed input (fp32 or its bf16 copy): one launch per sublayer boundary.
 """
 
 from __future__ import annotations
@@ -33,7 +38,8 @@ import torch.nn as nn
 
 from lit_gpt import seq_ops
 from lit_gpt.config import LayeredConfig, LayerSpec
-from lit_gpt.mixers import MIXERS, GatedFeedForward, SparseFeedForward, StepBatch, StreamLinks, TokenSide
+from lit_gpt.mixers import (MIXERS, DenseFeedForward, GatedFeedForward, SparseFeedForward, StepBatch, StreamLinks,
+                            TokenSide)
 from lit_gpt.rmsnorm import StreamRMSNorm
 
 
@@ -214,13 +220,108 @@ class PostNormBlock(nn.Module):
         return [self.sub1] if self.sub2 is None else [self.sub1, self.sub2]
 
 
+class SandwichSublayer(nn.Module):
+    """One sublayer of a sandwich layer: the input norm's weight, the fused input projection of everything that reads
+    the normed input (none when the module makes its own product), the module, and the output norm's weight times the
+    layer's per-channel scale (folded once, in fp32)."""
+
+    def __init__(self, module: nn.Module, norm_w: torch.Tensor, post_w: torch.Tensor, scale: Optional[torch.Tensor],
+                 width: int, device, dtype) -> None:
+        super().__init__()
+        self.module = module
+        for t in (norm_w, post_w) + ((scale,) if scale is not None else ()):
+            if t.numel() != width:
+                raise ValueError("norm / layer scale: one value per channel of the model's width")
+        self.register_buffer("norm_w", norm_w.to(device=device, dtype=torch.float32).contiguous())
+        post = post_w.to(device=device, dtype=torch.float32)
+        if scale is not None:
+            post = post * scale.to(device=device, dtype=torch.float32)
+        self.register_buffer("post_w", post.contiguous())
+        self.register_buffer("w_in", None)
+        parts = module.in_parts()
+        if parts:
+            self.w_in, offsets = _fuse_rows(parts, width, device, dtype)
+            module.bind(offsets)
+
+    def wants_bf16(self, rows: int) -> bool:
+        """Whether the norm that feeds this sublayer should leave a bf16 copy (bf16 MFMA tiles read it)."""
+        return rows > 8 and self._dtype() == torch.bfloat16
+
+    def _dtype(self):
+        return self.w_in.dtype if self.w_in is not None else self.module.w_up.dtype
+
+    def forward(self, h: Optional[torch.Tensor], h16: Optional[torch.Tensor], step: StepBatch, cache):
+        """h / h16 (T, width): the normed input (fp32 and / or its bf16 copy). Returns (branches, factor): the
+        sublayer's output as one (y, None) pair, or a two-branch mixer's (y, weight) pairs, for the boundary launch."""
+        src = h16 if h16 is not None else h
+        T, W = src.shape
+        proj = None
+        if self.w_in is not None and self.module.wants_proj(T):
+            n_in = self.w_in.shape[0]
+            proj = torch.empty(T, n_in, dtype=torch.float32, device=src.device)
+            seq_ops.linear(src, self.w_in, M=T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
+        y = torch.empty(T, W, dtype=torch.float32, device=src.device)
+        if cache is None:
+            self.module(proj, h, y, h16=h16, accumulate=False)
+        elif getattr(self.module, "branch_norm", False):
+            return self.module.branches(proj, step, cache, y)
+        else:
+            self.module(proj, step, cache, y, accumulate=False)
+        return [(y, None)], 1.0
+
+
+class SandwichBlock(nn.Module):
+    """x <- x + ls1 * norm1b(mixer(norm1 x)), then x <- x + ls2 * norm2b(ff(norm2 x)) when the layer has a feed-forward."""
+
+    def __init__(self, index: int, spec: LayerSpec, config: LayeredConfig, w: Dict[str, torch.Tensor], device,
+                 dtype) -> None:
+        super().__init__()
+        W, eps, design = config.width, config.norm_eps, config.design
+        if design.norm != "rms" or design.norm_offset != 0.0:
+            raise NotImplementedError("sandwich layers use RMS norms with plain weights")
+        self.mixer = MIXERS[spec.mixer.kind](spec.mixer, W, eps, _sub(w, "mix."), device, dtype)
+        self.sub1 = SandwichSublayer(self.mixer, w["norm1"], w["norm1b"], w.get("ls1"), W, device, dtype)
+        self.sub2 = None
+        if spec.mlp is not None:
+            if spec.mlp.kind == "dense":
+                if design.dense_ff != "relu2":
+                    raise NotImplementedError("sandwich layers serve the ungated relu^2 feed-forward")
+                mlp = DenseFeedForward(spec.mlp, W, _sub(w, "mlp."), device, dtype)
+            else:
+                mlp = SparseFeedForward(spec.mlp, W, _sub(w, "mlp."), device, dtype, route=design.moe)
+            self.sub2 = SandwichSublayer(mlp, w["norm2"], w["norm2b"], w.get("ls2"), W, device, dtype)
+
+    def sublayers(self) -> List[SandwichSublayer]:
+        return [self.sub1] if self.sub2 is None else [self.sub1, self.sub2]
+
+
 def _mixer_shapes(p: str, m, W: int) -> Dict[str, Tuple[int, ...]]:
     """Name -> shape of the tensors of a gated delta rule, a sink attention or a pair of them under prefix p."""
     if m.kind == "parallel":
-        return {**_mixer_shapes(p + "left.", m.left, W), **_mixer_shapes(p + "right.", m.right, W)}
-    if m.kind == "sink_attention":
-        return {p + "q": (m.heads * m.dim, W), p + "k": (m.kv_heads * m.dim, W), p + "v": (m.kv_heads * m.vdim, W),
-                p + "sink": (m.heads,), p + "o": (W, m.heads * m.vdim)}
+        out = {**_mixer_shapes(p + "left.", m.left, W), **_mixer_shapes(p + "right.", m.right, W)}
+        if m.branch_norm:
+            out.update({p + "left.out": (W,), p + "right.out": (W,)})
+        return out
+    if m.kind in ("sink_attention", "rotary_attention", "key_value_attention"):
+        out = {p + "q": (m.heads * m.dim, W), p + "k": (m.kv_heads * m.dim, W), p + "o": (W, m.heads * m.vdim)}
+        if m.values == "own":
+            out[p + "v"] = (m.kv_heads * m.vdim, W)
+        if m.sink_kind == "learned":
+            out[p + "sink"] = (m.heads,)
+        if m.qk_norm == "weight":
+            out.update({p + "q.norm": (m.dim,), p + "k.norm": (m.dim,)})
+        if m.head_gate:
+            out[p + "g"] = (m.heads, W)
+        return out
+    if m.kind in ("gated_linear", "lightning"):
+        qk, v = m.heads * m.dim, m.heads * m.vdim
+        out = {p + "q": (qk, W), p + "k": (qk, W), p + "v": (v, W), p + "g": (v, W), p + "o": (W, v)}
+        if m.kind == "gated_linear":
+            rank = m.decay_rank or 16
+            out.update({p + "norm": (m.vdim,), p + "a1": (rank, W), p + "a2": (qk, rank), p + "a2.b": (qk,)})
+        else:
+            out[p + "norm"] = (v,)
+        return out
     qk, v = m.kv_heads * m.dim, m.heads * m.vdim
     out = {p + "q": (qk, W), p + "q.conv": (qk, m.conv), p + "k": (qk, W), p + "k.conv": (qk, m.conv), p + "v": (v, W),
            p + "v.conv": (v, m.conv), p + "b": (m.heads, W), p + "A_log": (m.heads,), p + "norm": (m.vdim,),
@@ -258,6 +359,7 @@ class LayeredGPT(nn.Module):
         design = config.design
         self.sequential = design.block == "sequential"
         self.post = design.block == "post"
+        self.sandwich = design.block == "sandwich"
         self.register_buffer("pos_table", None)
         if design.positions == "learned":
             t = weights["pos"]
@@ -268,6 +370,11 @@ class LayeredGPT(nn.Module):
             if config.side_dim or config.streams != 1:
                 raise NotImplementedError("post-norm layers have one residual stream and no per-layer token input")
             self.blocks = nn.ModuleList(PostNormBlock(i, spec, config, _sub(weights, f"l{i}."), device, dtype)
+                                        for i, spec in enumerate(config.layers))
+        elif self.sandwich:
+            if config.side_dim or config.streams != 1:
+                raise NotImplementedError("sandwich layers have one residual stream and no per-layer token input")
+            self.blocks = nn.ModuleList(SandwichBlock(i, spec, config, _sub(weights, f"l{i}."), device, dtype)
                                         for i, spec in enumerate(config.layers))
         elif self.sequential:
             if config.side_dim:
@@ -328,6 +435,10 @@ class LayeredGPT(nn.Module):
             out[p + "norm1"] = (W,)
             if spec.mlp is not None and config.design.block != "parallel":
                 out[p + "norm2"] = (W,)
+            if config.design.block == "sandwich":
+                out.update({p + "norm1b": (W,), p + "ls1": (W,)})
+                if spec.mlp is not None:
+                    out.update({p + "norm2b": (W,), p + "ls2": (W,)})
             if biased:
                 out.update({name + ".b": (W,) for name in (p + "norm1", p + "norm2") if name in out})
             if config.stream_weights:
@@ -343,7 +454,8 @@ class LayeredGPT(nn.Module):
                 if m.kv_from is None:
                     out.update({p + "mix.k": (2 * m.kv_heads * m.dim, W), p + "mix.v": (m.kv_heads * m.vdim, W)})
                 out.update({p + f"mix.{n}": (m.dim,) for n in ("lq1", "lk1", "lq2", "lk2")})
-            elif m.kind in ("channel_delta", "gated_delta", "sink_attention", "parallel"):
+            elif m.kind in ("channel_delta", "gated_delta", "sink_attention", "parallel", "rotary_attention",
+                            "key_value_attention", "gated_linear", "lightning"):
                 out.update(_mixer_shapes(p + "mix.", m, W))
             elif m.kind == "mamba2":
                 inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
@@ -356,7 +468,9 @@ class LayeredGPT(nn.Module):
                             p + "mix.uv": (m.heads * m.vdim, m.kv_rank), p + "mix.sink": (m.heads,),
                             p + "mix.g": (m.heads * m.vdim, W), p + "mix.o": (W, m.heads * m.vdim)})
             f = spec.mlp
-            if f is not None and f.kind == "dense":
+            if f is not None and f.kind == "dense" and config.design.dense_ff == "relu2":
+                out.update({p + "mlp.up": (f.ff, W), p + "mlp.down": (W, f.ff)})
+            elif f is not None and f.kind == "dense":
                 out.update({p + "mlp.gate": (f.ff, W), p + "mlp.up": (f.ff, W), p + "mlp.down": (W, f.ff)})
             elif f is not None:
                 gated = config.design.moe == "scores"
@@ -367,6 +481,9 @@ class LayeredGPT(nn.Module):
                     if gated:
                         out[p + f"mlp.e{e}.gate"] = (f.ff, W)
                     out.update({p + f"mlp.e{e}.up": (f.ff, W), p + f"mlp.e{e}.down": (W, f.ff)})
+                if f.shared_ff:
+                    out.update({p + "mlp.shared.up": (f.shared_ff, W), p + "mlp.shared.down": (W, f.shared_ff),
+                                p + "mlp.shared.sg": (1, W)})
             if config.side_dim:
                 out.update({p + "side.gate": (config.side_dim, W), p + "side.proj": (W, config.side_dim),
                             p + "side.norm": (W,)})
@@ -381,8 +498,14 @@ class LayeredGPT(nn.Module):
         neutral = 1.0 - config.design.norm_offset
         for name, shape in cls.tensor_shapes(config).items():
             leaf = name.rsplit(".", 1)[-1]
-            if leaf in ("norm1", "norm2") or name == "final.norm":
+            if leaf in ("norm1", "norm2", "norm1b", "norm2b") or name == "final.norm":
                 t = neutral + 0.1 * torch.randn(shape, generator=g)
+            elif leaf in ("ls1", "ls2"):
+                t = 0.5 + 0.2 * torch.randn(shape, generator=g)
+            elif name.endswith((".left.out", ".right.out", "q.norm", "k.norm")):
+                t = 1.0 + 0.2 * torch.randn(shape, generator=g)
+            elif name.endswith("a2.b"):
+                t = 2.0 + torch.randn(shape, generator=g)
             elif name.endswith(("norm1.b", "norm2.b", "final.norm.b", "correction")):
                 t = 0.1 * torch.randn(shape, generator=g)
             elif name == "pos":
@@ -469,6 +592,8 @@ class LayeredGPT(nn.Module):
             return self._forward_streams(step)
         if self.post:
             return self._forward_post(step)
+        if self.sandwich:
+            return self._forward_sandwich(step)
         x = seq_ops.embed(step.tokens, self.embed, self.config.embedding_scale)
         for run, layer in enumerate(self.runs):
             self.blocks[layer](x, step, self.caches[run])
@@ -490,6 +615,33 @@ class LayeredGPT(nn.Module):
                                         bf16_copy=want16)
                 x16 = got[1] if want16 else None
             if after_layer is not None:
+                after_layer(run, x)
+        return x
+
+    def _forward_sandwich(self, step: StepBatch, after_layer=None) -> torch.Tensor:
+        """The sandwich layers. Every boundary between two sublayers is one launch: the branch norms and the average of
+        a two-branch mixer, the output norm times the layer scale, the residual add, and the next sublayer's normed
+        input (for more than 8 rows with bf16 weights only its bf16 copy, unless the next module also reads it in
+        fp32). ``after_layer(run, x)``: a hook that sees the residual (T, width) after each layer run (for tests)."""
+        eps = self.config.norm_eps
+        x = seq_ops.embed(step.tokens, self.embed, self.config.embedding_scale)
+        chain = [(run, sub, self.caches[run] if k == 0 else None)
+                 for run, layer in enumerate(self.runs) for k, sub in enumerate(self.blocks[layer].sublayers())]
+
+        def reads(sub):  # (fp32 input wanted, bf16 copy wanted)
+            b16 = sub.wants_bf16(step.T)
+            return (not b16) or getattr(sub.module, "reads_f32", False), b16
+
+        f32, b16 = reads(chain[0][1])
+        h, h16 = seq_ops.sandwich_step(x, next_w=chain[0][1].norm_w, eps=eps, want_f32=f32, bf16_copy=b16)
+        for n, (run, sub, cache) in enumerate(chain):
+            branches, coef = sub(h, h16, step, cache)
+            nxt = chain[n + 1][1] if n + 1 < len(chain) else None
+            f32, b16 = reads(nxt) if nxt is not None else (False, False)
+            h, h16 = seq_ops.sandwich_step(x, branches=branches, coef=coef, post_w=sub.post_w,
+                                           next_w=nxt.norm_w if nxt is not None else None, eps=eps, want_f32=f32,
+                                           bf16_copy=b16)
+            if after_layer is not None and (nxt is None or chain[n + 1][0] != run):
                 after_layer(run, x)
         return x
 

@@ -90,14 +90,26 @@ class Retention(InputReader):
     """A per-head outer-product memory with a constant decay, read by the query (linear attention, scores neither
     normalised nor soft-maxed): per head S_t = decay S_{t-1} + k_t v_t^T,
     o_t = S_t^T q_t, rotary positions (pairs i, i + dims/2) on q and k, k scaled by ``k_scale``; each head's output is
-    divided by its root mean square, gated with silu(W_g h) and projected."""
+    divided by its root mean square, gated with silu(W_g h) and projected.
 
-    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+    Options (the "lightning" kind sets them): ``act`` an activation on q, k and v as projected; ``k_scale`` (default
+    dim^-1/2); ``joint_norm`` the concatenated heads are RMS-normed together with the weight ``norm`` (H dv values)
+    instead of head by head without one; ``gate_act`` the gate's activation."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype, *,
+                 act: int = seq_ops.ACT_NONE, k_scale: Optional[float] = None, joint_norm: bool = False,
+                 gate_act: int = seq_ops.ACT_SILU) -> None:
         super().__init__()
         self.H, self.d, self.dv, self.eps = spec.heads, spec.dim, spec.vdim, eps
         self.rot_dims = spec.rot.dims
-        self.k_scale = float(spec.dim) ** -0.5
+        self.k_scale = float(spec.dim) ** -0.5 if k_scale is None else float(k_scale)
+        self.act, self.joint_norm, self.gate_act = act, joint_norm, gate_act
         H, d, dv = self.H, self.d, self.dv
+        self.register_buffer("norm_w", None)
+        if joint_norm:
+            if w["norm"].numel() != H * dv:
+                raise ValueError(f"{spec.kind}.norm: {w['norm'].numel()} values, expected {H * dv}")
+            self.norm_w = _f32(w["norm"], device)
         for name, rows in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv)):
             if tuple(w[name].shape) != (rows, width):
                 raise ValueError(f"retention.{name}: shape {tuple(w[name].shape)}, expected {(rows, width)}")
@@ -114,13 +126,19 @@ class Retention(InputReader):
         return RetentionState(slots, self.H, self.d, self.dv, device=device)
 
     def forward(self, proj: torch.Tensor, step: StepBatch, cache: RetentionState, x: torch.Tensor,
-                accumulate: bool = True) -> None:
+                accumulate: bool = True, post: float = 1.0) -> None:
         H, dv = self.H, self.dv
         o = seq_ops.retention(proj, self.off["q"], self.off["k"], self.off["v"], cache.s, self.decay, self.inv_freq,
                               step.seq_start, step.seq_slot, step.seq_pos0, H=H, d=self.d, dv=dv,
-                              rot_dims=self.rot_dims, k_scale=self.k_scale, max_len=step.max_len, pos=step.pos)
-        o = seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU,
-                              bf16_copy=_tiles16(step.T, self.w_o))
+                              rot_dims=self.rot_dims, k_scale=self.k_scale, max_len=step.max_len, pos=step.pos,
+                              act=self.act)
+        if self.joint_norm:  # one "head" of H dv values with a weight
+            o = seq_ops.head_gate(o, proj, self.off["g"], H=1, dv=H * dv, unit_norm=True, eps=self.eps,
+                                  act=self.gate_act, weight=self.norm_w, post=post,
+                                  bf16_copy=_tiles16(step.T, self.w_o))
+        else:
+            o = seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=self.gate_act,
+                                  post=post, bf16_copy=_tiles16(step.T, self.w_o))
         W = x.shape[1]
         seq_ops.linear(o, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
 
@@ -385,21 +403,48 @@ class SinkAttention(InputReader):
     mean square per head (no weight), the query is multiplied by a temperature that grows with its position,
     1 + coef * ln(floor((p + 1) / every) + 1); score = (q . k) * scale; a learned per-head sink scalar adds its
     exponential to the softmax normaliser without contributing a value. The cache holds the normed keys and the
-    values."""
+    values.
+
+    The spec's options make its relatives: ``qk_norm`` "none" / "unit" / "weight" (times ``q.norm`` / ``k.norm``, d
+    values shared by the heads); rotary positions on the pairs (i, i + rot.dims / 2) of the first ``rot.dims`` dims
+    after the norm (frequencies optionally rescaled band by band); ``sink_kind`` "none" / "learned" / "one" (a sink of
+    score 0: the denominator is 1 + sum exp); ``values`` "keys": no value projection, the values are the keys as
+    projected, before their norm; ``head_gate``: head h's output times sigmoid(W_g h)_h, one number per head."""
 
     def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
         super().__init__()
         self.H, self.G, self.d, self.dv, self.eps = spec.heads, spec.kv_heads, spec.dim, spec.vdim, eps
         self.scale, self.cap, self.chunk = spec.scale, spec.softcap, spec.mask_size
         self.temp_coef, self.temp_every = spec.q_temp_coef, spec.q_temp_every
+        self.qk_norm, self.own_values, self.head_gate = spec.qk_norm, spec.values == "own", spec.head_gate
+        self.rot_dims = spec.rot.dims
         H, G, d, dv = self.H, self.G, self.d, self.dv
-        for name, shape in (("q", (H * d, width)), ("k", (G * d, width)), ("v", (G * dv, width)), ("o", (width, H * dv))):
+        shapes = [("q", (H * d, width)), ("k", (G * d, width)), ("o", (width, H * dv))]
+        shapes += [("v", (G * dv, width))] if self.own_values else []
+        shapes += [("g", (H, width))] if self.head_gate else []
+        for name, shape in shapes:
             if tuple(w[name].shape) != shape:
-                raise ValueError(f"sink_attention.{name}: shape {tuple(w[name].shape)}, expected {shape}")
-        if "sink" in w and w["sink"].numel() != H:
-            raise ValueError(f"sink_attention.sink: {w['sink'].numel()} values, expected {H}")
-        self._in = [(n, w[n]) for n in ("q", "k", "v")]
-        self.register_buffer("sink", _f32(w["sink"], device) if "sink" in w else None)
+                raise ValueError(f"{spec.kind}.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        if not self.own_values and dv != d:
+            raise ValueError(f"{spec.kind}: values that are the keys have the keys' size")
+        self._in = [(n, w[n]) for n in (("q", "k", "v") if self.own_values else ("q", "k"))]
+        self._in += [("g", w["g"])] if self.head_gate else []
+        self.register_buffer("sink", None)
+        if spec.sink_kind == "one":
+            self.sink = torch.zeros(H, dtype=torch.float32, device=device)
+        elif spec.sink_kind == "learned" and "sink" in w:
+            if w["sink"].numel() != H:
+                raise ValueError(f"{spec.kind}.sink: {w['sink'].numel()} values, expected {H}")
+            self.sink = _f32(w["sink"], device)
+        self.register_buffer("q_norm", None)
+        self.register_buffer("k_norm", None)
+        if self.qk_norm == "weight":
+            if w["q.norm"].numel() != d or w["k.norm"].numel() != d:
+                raise ValueError(f"{spec.kind}: q.norm / k.norm hold {d} values")
+            self.q_norm, self.k_norm = _f32(w["q.norm"], device), _f32(w["k.norm"], device)
+        self.register_buffer("inv_freq", None)
+        if self.rot_dims > 0:
+            self.inv_freq = torch.tensor(spec.rot.inv_freq(), dtype=torch.float64).to(device=device, dtype=torch.float32)
         self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
 
     def in_parts(self):
@@ -411,24 +456,90 @@ class SinkAttention(InputReader):
     def forward(self, proj: torch.Tensor, step: StepBatch, cache: HeadKVCache, x: torch.Tensor, accumulate: bool = True,
                 post: float = 1.0) -> None:
         H, G, d, dv = self.H, self.G, self.d, self.dv
-        seq_ops.normattn_prepare(proj, self.off["q"], self.off["k"], self.off["v"], cache.k, cache.v, step.slot,
-                                 step.pos, H=H, G=G, d=d, dv=dv, eps=self.eps, temp_coef=self.temp_coef,
-                                 temp_every=self.temp_every)
+        seq_ops.normattn_prepare(proj, self.off["q"], self.off["k"], self.off["v" if self.own_values else "k"], cache.k,
+                                 cache.v, step.slot, step.pos, H=H, G=G, d=d, dv=dv, eps=self.eps,
+                                 temp_coef=self.temp_coef, temp_every=self.temp_every, norm=self.qk_norm != "none",
+                                 q_weight=self.q_norm, k_weight=self.k_norm, inv_freq=self.inv_freq,
+                                 rot_dims=self.rot_dims)
         att = seq_ops.sinkattn(proj, self.off["q"], cache.k, cache.v, self.sink, step.seq_start, step.seq_slot,
                                step.seq_pos0, step.max_len or step.T, H=H, G=G, d=d, dv=dv, scale=self.scale,
-                               chunk=self.chunk, cap=self.cap, post=post, bf16_copy=_tiles16(step.T, self.w_o))
+                               chunk=self.chunk, cap=self.cap, post=post, bf16_copy=_tiles16(step.T, self.w_o),
+                               gate_off=self.off["g"] if self.head_gate else -1)
         W = x.shape[1]
         seq_ops.linear(att, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
 
 
+class GatedLinearAttention(InputReader):
+    """Linear attention with a decay per head and key channel and no correction towards the key's value: per head
+    S <- diag(alpha) S + k v^T, o = S^T q (the state S is dim x vdim, fp32, in a cache slot), q = W_q h * dim^-1/2,
+    alpha = sigmoid(W_a2 (W_a1 h) + b)^(1 / tau) (a low-rank pair of maps with a bias). Each head's output is RMS-normed
+    over vdim with one weight vector for all heads, multiplied by silu(W_g h) and projected. The recurrence is the gated
+    delta rule's kernel without its correction, token by token in every step kind."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        self.H, self.d, self.dv, self.eps, self.tau = spec.heads, spec.dim, spec.vdim, eps, float(spec.tau)
+        H, d, dv = self.H, self.d, self.dv
+        rank = w["a1"].shape[0]
+        for name, shape in (("q", (H * d, width)), ("k", (H * d, width)), ("v", (H * dv, width)), ("g", (H * dv, width)),
+                            ("a1", (rank, width)), ("a2", (H * d, rank)), ("a2.b", (H * d,)), ("norm", (dv,)),
+                            ("o", (width, H * dv))):
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"{spec.kind}.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        self._in = [("qkv", torch.cat([w["q"], w["k"], w["v"]])), ("g", w["g"]), ("a1", w["a1"])]
+        self.register_buffer("w_a2", w["a2"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("a_bias", _f32(w["a2.b"], device))
+        self.register_buffer("norm_w", _f32(w["norm"], device))
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> RetentionState:
+        return RetentionState(slots, self.H, self.d, self.dv, device=device)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: RetentionState, x: torch.Tensor,
+                accumulate: bool = True, post: float = 1.0) -> None:
+        H, d, dv = self.H, self.d, self.dv
+        T, ld = proj.shape
+        rank = self.w_a2.shape[1]
+        kw = dict(H=H, G=H, d=d, per_channel=True, q_scale=float(d) ** -0.5, unit=False, decay_form=1, tau=self.tau,
+                  qkv_off=self.off["qkv"])
+        if T <= 8 and rank <= 512:  # few tokens: the second map of the decay inside the preparation launch
+            dec, _, kq = seq_ops.delta_prepare(proj, proj, self.off["a1"], None, 0, None, self.a_bias, w_a2=self.w_a2, **kw)
+        else:
+            a = torch.empty(T, H * d, dtype=torch.float32, device=proj.device)
+            seq_ops.linear(proj, self.w_a2, M=T, N=H * d, K=rank, y=a, a_off=self.off["a1"], lda=ld, ldy=H * d)
+            dec, _, kq = seq_ops.delta_prepare(proj, a, 0, None, 0, None, self.a_bias, **kw)
+        o = seq_ops.gated_delta(proj, dec, None, kq, cache.s, step.seq_start, step.seq_slot, step.seq_pos0, H=H, G=H,
+                                d=d, dv=dv, per_channel=True, plain=True, qkv_off=self.off["qkv"])
+        o = seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU,
+                              weight=self.norm_w, post=post, bf16_copy=_tiles16(T, self.w_o))
+        W = x.shape[1]
+        seq_ops.linear(o, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
+
+
+class Lightning(Retention):
+    """The constant-decay rule on activated projections: q = silu(W_q h), k = silu(W_k h), v = silu(W_v h), per head
+    S <- decay_h S + k v^T, o = S^T q (no rotation, no key scale); the concatenated heads are RMS-normed together with
+    the weight ``norm``, multiplied by sigmoid(W_g h) and projected."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__(spec, width, eps, w, device, dtype, act=seq_ops.ACT_SILU, k_scale=1.0, joint_norm=True,
+                         gate_act=seq_ops.ACT_SIGMOID)
+
+
 class ParallelMixer(InputReader):
-    """Two mixers side by side on the same input, summed with fixed factors: ``left_scale`` * a sink attention
-    (tensors under ``left.``) + ``right_scale`` * a gated delta rule with one decay per head (``right.``). Both read
-    the layer's one input projection; each factor is applied where its mixer's last elementwise kernel runs, and the
-    second out-projection accumulates onto the first. With ``overlap`` the delta rule's kernels of a prompt step run
-    on a second HIP stream (default priority) beside the attention's: they touch disjoint columns of the projection
-    and different caches; the second stream starts after the projection and is joined before the delta rule's
-    out-projection."""
+    """Two mixers side by side on the same input (tensors under ``left.`` and ``right.``; which kinds, the spec says:
+    a sink attention beside a gated delta rule, a rotary attention beside a gated linear attention, ...). Both read
+    the layer's one input projection. Plain form: ``left_scale`` * left + ``right_scale`` * right, each factor applied
+    where its mixer's last elementwise kernel runs, the second out-projection accumulating onto the first. With
+    ``branch_norm`` each branch's output is first RMS-normed over the width with its own weight (``left.out`` /
+    ``right.out``): the branches then go to buffers of their own and ``branches()`` hands them, with the weights, to the
+    layer's norm + residual launch, which also forms the weighted sum. With ``overlap`` the right mixer's kernels of a
+    prompt step run on a second HIP stream (default priority) beside the left's: they touch disjoint columns of the
+    projection and different caches; the second stream starts after the projection and is joined before the two
+    outputs meet."""
 
     overlap = True
     OVERLAP_ROWS = 8  # steps of up to this many rows stay on one stream (a captured one-token step gains nothing)
@@ -437,9 +548,18 @@ class ParallelMixer(InputReader):
     def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
         super().__init__()
         sub = lambda prefix: {k[len(prefix):]: v for k, v in w.items() if k.startswith(prefix)}  # noqa: E731
-        self.left = SinkAttention(spec.left, width, eps, sub("left."), device, dtype)
-        self.right = GatedDelta(spec.right, width, eps, sub("right."), device, dtype, per_channel=False)
+        self.left = MIXERS[spec.left.kind](spec.left, width, eps, sub("left."), device, dtype)
+        self.right = MIXERS[spec.right.kind](spec.right, width, eps, sub("right."), device, dtype)
         self.left_scale, self.right_scale = spec.left_scale, spec.right_scale
+        self.branch_norm = spec.branch_norm
+        self.register_buffer("left_out", None)
+        self.register_buffer("right_out", None)
+        if self.branch_norm:
+            if spec.left_scale != spec.right_scale:
+                raise NotImplementedError("normed branches are summed with one common factor")
+            if w["left.out"].numel() != width or w["right.out"].numel() != width:
+                raise ValueError("parallel.left.out / right.out: one weight per channel of the model's width")
+            self.left_out, self.right_out = _f32(w["left.out"], device), _f32(w["right.out"], device)
 
     def in_parts(self):
         return [("left." + n, t) for n, t in self.left.in_parts()] + [("right." + n, t) for n, t in self.right.in_parts()]
@@ -452,17 +572,40 @@ class ParallelMixer(InputReader):
         return CachePair(self.left.build_cache(slots, max_seq_length, device, dtype),
                          self.right.build_cache(slots, max_seq_length, device, dtype))
 
+    def _side_stream(self, device) -> "torch.cuda.Stream":
+        index = device.index or 0
+        side = self._side.get(index)
+        if side is None:
+            side = self._side[index] = torch.cuda.Stream(device=device)
+        return side
+
+    def branches(self, proj: torch.Tensor, step: StepBatch, cache: CachePair, y: torch.Tensor):
+        """The normed form: the left mixer's output goes to ``y``, the right's to a buffer of its own; returns
+        ([(y_left, w_left), (y_right, w_right)], common factor) for the layer's norm + residual launch."""
+        yr = torch.empty_like(y)
+        if not self.overlap or step.T <= self.OVERLAP_ROWS:
+            self.left(proj, step, cache.left, y, accumulate=False)
+            self.right(proj, step, cache.right, yr, accumulate=False)
+        else:
+            main = torch.cuda.current_stream(proj.device)
+            side = self._side_stream(proj.device)
+            side.wait_stream(main)  # the projection is made
+            with torch.cuda.stream(side):
+                self.right(proj, step, cache.right, yr, accumulate=False)
+            self.left(proj, step, cache.left, y, accumulate=False)
+            main.wait_stream(side)
+        return [(y, self.left_out), (yr, self.right_out)], self.left_scale
+
     def forward(self, proj: torch.Tensor, step: StepBatch, cache: CachePair, x: torch.Tensor,
                 accumulate: bool = True) -> None:
-        if not self.overlap or step.T <= self.OVERLAP_ROWS:
+        if self.branch_norm:
+            raise RuntimeError("normed branches meet in the layer's norm launch: call branches()")
+        if not self.overlap or step.T <= self.OVERLAP_ROWS or not hasattr(self.right, "mix"):
             self.left(proj, step, cache.left, x, accumulate=accumulate, post=self.left_scale)
             self.right(proj, step, cache.right, x, accumulate=True, post=self.right_scale)
             return
         main = torch.cuda.current_stream(proj.device)
-        index = proj.device.index or 0
-        side = self._side.get(index)
-        if side is None:
-            side = self._side[index] = torch.cuda.Stream(device=proj.device)
+        side = self._side_stream(proj.device)
         side.wait_stream(main)  # the projection is made
         with torch.cuda.stream(side):
             o = self.right.mix(proj, step, cache.right, post=self.right_scale)
@@ -520,6 +663,39 @@ class GatedFeedForward(InputReader):
         seq_ops.linear(a, self.w_down, M=a.shape[0], N=W, K=self.ff, y=x, lda=self.ff, ldy=W, accumulate=accumulate)
 
 
+class DenseFeedForward(InputReader):
+    """W_down act(W_up h) without a gate (``act`` defaults to the square of relu). The unit is the only reader of its
+    input, so it makes the up product itself, with the activation in the product's epilogue (for MFMA tiles the
+    result is left in bf16, the down product's operand)."""
+
+    def __init__(self, spec: FeedForwardSpec, width: int, w: Dict[str, torch.Tensor], device, dtype,
+                 act: int = seq_ops.ACT_RELU2) -> None:
+        super().__init__()
+        self.ff, self.act = spec.ff, act
+        for name, shape in (("up", (spec.ff, width)), ("down", (width, spec.ff))):
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"mlp.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        self.register_buffer("w_up", w["up"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("w_down", w["down"].to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return []
+
+    def wants_proj(self, rows: int) -> bool:
+        return False
+
+    def forward(self, proj, h: Optional[torch.Tensor], x: torch.Tensor, h16: Optional[torch.Tensor] = None,
+                accumulate: bool = True) -> None:
+        """h: the normed input in fp32, or None when only its bf16 copy ``h16`` was made (MFMA tiles)."""
+        T, W = x.shape
+        F = self.ff
+        bf16 = _tiles16(T, self.w_down)
+        src = h16 if (bf16 and h16 is not None) else h
+        a = torch.empty(T, F, dtype=torch.bfloat16 if bf16 else torch.float32, device=x.device)
+        seq_ops.linear(src, self.w_up, M=T, N=F, K=W, y=a, lda=W, ldy=F, act=self.act)
+        seq_ops.linear(a, self.w_down, M=T, N=W, K=F, y=x, lda=F, ldy=W, accumulate=accumulate)
+
+
 class SparseFeedForward(InputReader):
     """Mixture of experts with an fp32 router, in one of two forms.
 
@@ -529,25 +705,43 @@ class SparseFeedForward(InputReader):
     (a stored vector that shifts the choice only) are chosen; the weights are the chosen scores as they are;
     expert = W_down (act(W_gate h) * W_up h) (``act`` defaults to silu); the last ``identity`` router outputs are
     identity experts without matrices, whose output is the input itself.
+    ``route = "sigmoid"``: scores = sigmoid of every router output on its own; the ``top`` largest are chosen; the
+    chosen score multiplies the expert's INPUT, expert = W_down relu(W_up (s h))^2. Since s > 0 that equals
+    s^2 W_down relu(W_up h)^2, which is what runs: the routing launch hands out s^2 as the weight of the expert's
+    output (another activation than the square of relu is refused). With ``shared_ff`` a shared expert of the same
+    form (``shared.up`` / ``shared.down``) runs for every token and is added times sigmoid(W_sg h), one number per
+    token (``shared.sg``); its up matrix, its gate row and the router are one fused input projection.
 
     Few (token, choice) pairs (decode) stream only the chosen experts' rows through two GEMV launches. A prompt
     sorts its pairs by expert on the device and runs two grouped products over the expert ranges, then sums each
     token's choices in routing order."""
 
     STREAM_PAIRS = 48  # up to this many (token, choice) pairs the streaming form runs
+    reads_f32 = True  # the streaming experts and the in-launch router read the fp32 input itself
 
     def __init__(self, spec: FeedForwardSpec, width: int, w: Dict[str, torch.Tensor], device, dtype,
                  act: Optional[int] = None, route: str = "top_logits") -> None:
         super().__init__()
-        if route not in ("top_logits", "scores"):
+        if route not in ("top_logits", "scores", "sigmoid"):
             raise ValueError(f"unknown routing {route!r}")
         self.E, self.top, self.ff, self.route = spec.experts, spec.top, spec.ff, route
         self.gated = route == "scores"
         self.n_router = spec.experts + (spec.identity if self.gated else 0)
         self.act = act if act is not None else (seq_ops.ACT_SILU if self.gated else seq_ops.ACT_RELU2)
+        if route == "sigmoid" and self.act != seq_ops.ACT_RELU2:
+            raise NotImplementedError("a score on the expert's input is served for the square of relu")
+        self.shared_ff = spec.shared_ff if route == "sigmoid" else 0
         if tuple(w["router"].shape) != (self.n_router, width):
             raise ValueError(f"mlp.router: shape {tuple(w['router'].shape)}, expected {(self.n_router, width)}")
         self._in = [("router", w["router"])]
+        self.register_buffer("w_shared_down", None)
+        if self.shared_ff:
+            Fs = self.shared_ff
+            for name, shape in (("shared.up", (Fs, width)), ("shared.down", (width, Fs)), ("shared.sg", (1, width))):
+                if tuple(w[name].shape) != shape:
+                    raise ValueError(f"mlp.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+            self._in += [("shared.up", w["shared.up"]), ("shared.sg", w["shared.sg"])]
+            self.w_shared_down = w["shared.down"].to(device=device, dtype=dtype).contiguous()
         up = torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) if self.gated else w[f"e{e}.up"]
                           for e in range(self.E)])
         down = torch.stack([w[f"e{e}.down"] for e in range(self.E)])
@@ -557,7 +751,8 @@ class SparseFeedForward(InputReader):
         self.register_buffer("w_up", up.to(device=device, dtype=dtype).contiguous())  # gated: gate rows, then up rows
         self.register_buffer("w_down", down.to(device=device, dtype=dtype).contiguous())
         # (steps with few tokens compute the router's logits inside the routing launch, from this copy)
-        self.register_buffer("w_router", w["router"].to(device=device, dtype=dtype).contiguous() if self.gated else None)
+        fused_router = self.gated or (route == "sigmoid" and not self.shared_ff)
+        self.register_buffer("w_router", w["router"].to(device=device, dtype=dtype).contiguous() if fused_router else None)
         self.register_buffer("correction", None)
         if self.gated and "correction" in w:
             if w["correction"].numel() != self.n_router:
@@ -569,7 +764,7 @@ class SparseFeedForward(InputReader):
 
     def wants_proj(self, rows: int) -> bool:
         """Whether a step of ``rows`` tokens needs the layer's input projection (the router logits) made for it."""
-        return not (self.gated and rows * self.top <= self.STREAM_PAIRS)
+        return not (self.w_router is not None and rows * self.top <= self.STREAM_PAIRS)
 
     def forward(self, proj: Optional[torch.Tensor], h: torch.Tensor, x: torch.Tensor,
                 h16: Optional[torch.Tensor] = None, accumulate: bool = True) -> None:
@@ -577,8 +772,11 @@ class SparseFeedForward(InputReader):
         ``proj`` None (score routing, few tokens): the router's logits are made inside the routing launch."""
         T, W = h.shape
         E, top, F = self.E, self.top, self.ff
-        if self.gated and proj is None:
-            ids, wts = seq_ops.moe_router(h, self.w_router, top, self.correction)
+        sig = self.route == "sigmoid"
+        if proj is None:
+            ids, wts = seq_ops.moe_router(h, self.w_router, top, self.correction, sigmoid=sig, square=sig)
+        elif sig:
+            ids, wts = seq_ops.moe_route_scores(proj, self.off["router"], self.n_router, top, sigmoid=True, square=True)
         elif self.gated:
             ids, wts = seq_ops.moe_route_scores(proj, self.off["router"], self.n_router, top, self.correction)
         else:
@@ -586,6 +784,7 @@ class SparseFeedForward(InputReader):
         if T * top <= self.STREAM_PAIRS:
             a = seq_ops.moe_up(h, self.w_up, ids, self.act, gated=self.gated)
             seq_ops.moe_down(a, self.w_down, ids, wts, x, h, accumulate=accumulate)
+            self._shared(proj, x)
             return
         pairs = T * top
         z_start, tok_of, where = seq_ops.moe_sort(ids, self.n_router)
@@ -604,6 +803,18 @@ class SparseFeedForward(InputReader):
         identity = self.n_router > E
         seq_ops.moe_combine(y, where, wts, x, ids=ids if identity else None, n_real=E, h=h if identity else None,
                             accumulate=accumulate)
+        self._shared(proj, x)
+
+    def _shared(self, proj: Optional[torch.Tensor], x: torch.Tensor) -> None:
+        """x += sigmoid(W_sg h) * W_down act(W_up h) of the shared expert: the gate scales the activated rows (one
+        number per row), then the down product accumulates."""
+        if not self.shared_ff:
+            return
+        T, W = x.shape
+        Fs = self.shared_ff
+        a = seq_ops.act_rows(proj, self.off["shared.up"], Fs, self.act, gate_off=self.off["shared.sg"],
+                             bf16=_tiles16(T, self.w_shared_down))
+        seq_ops.linear(a, self.w_shared_down, M=T, N=W, K=Fs, y=x, lda=Fs, ldy=W, accumulate=True)
 
 
 class TokenSide(nn.Module):
@@ -626,4 +837,5 @@ class TokenSide(nn.Module):
 
 MIXERS = {"retention": Retention, "latent_attention": LatentAttention, "attention": DiffAttention,
           "mamba2": SelectiveScan, "channel_delta": GatedDelta, "gated_delta": GatedDelta,
-          "sink_attention": SinkAttention, "parallel": ParallelMixer}
+          "sink_attention": SinkAttention, "parallel": ParallelMixer, "rotary_attention": SinkAttention,
+          "key_value_attention": SinkAttention, "gated_linear": GatedLinearAttention, "lightning": Lightning}

@@ -35,15 +35,17 @@ SIGNATURES = {
     "lgs_embed": [_P, _P, _I, _F, _P, _I, _I, _I, _P],
     "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P, _P],
     "lgs_gather_rows": [_P, _P, _P, _I, _I, _P],
-    "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _P],
+    "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _I, _P],
     "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P, _F, _P, _P, _I, _I, _P],
     "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
     "lgs_latent_attention_tiles": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _I, _P],
     "lgs_moe_route": [_P, _L, _I, _I, _I, _P, _P, _P],
-    "lgs_moe_route_scores": [_P, _L, _I, _I, _I, _P, _P, _P, _P],
-    "lgs_moe_router": [_P, _L, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
+    "lgs_moe_route_scores": [_P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P],
+    "lgs_moe_router": [_P, _L, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
+    "lgs_act_rows": [_P, _L, _P, _L, _P, _I, _I, _I, _I, _P],
+    "lgs_sandwich_step": [_P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _F, _I, _I, _P],
     "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _L, _I, _P],
     "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
@@ -61,12 +63,15 @@ SIGNATURES = {
     "lgs_embed_pos": [_P, _P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],
     "lgs_layernorm": [_P, _P, _P, _F, _F, _I, _P, _P, _I, _I, _P],
     "lgs_softcap": [_P, _L, _F, _P],
-    "lgs_normattn_prepare": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P],
-    "lgs_sinkattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P],
-    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P, _I, _I, _P],
+    "lgs_normattn_prepare": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _P, _P,
+                             _I, _P],
+    "lgs_sinkattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P,
+                     _L, _P],
+    "lgs_delta_prepare": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P, _I, _I, _I, _I, _F,
+                          _P],
     "lgs_delta_step_prepare": [_P, _L, _P, _I, _I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                _I, _F, _F, _P, _I, _I, _P],
-    "lgs_gated_delta": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "lgs_gated_delta": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
 }
 _RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
 
@@ -191,13 +196,15 @@ def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
 def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor, decay: torch.Tensor,
               inv_freq: Optional[torch.Tensor], seq_start: torch.Tensor, seq_slot: torch.Tensor,
               seq_pos0: torch.Tensor, *, H: int, d: int, dv: int, rot_dims: int, k_scale: float,
-              chunked: Optional[bool] = None, max_len: int = 0, pos: Optional[torch.Tensor] = None) -> torch.Tensor:
+              chunked: Optional[bool] = None, max_len: int = 0, pos: Optional[torch.Tensor] = None,
+              act: int = ACT_NONE) -> torch.Tensor:
     """proj (T, ld) holds q, k (H * d each) and v (H * dv) at the given column offsets; state (slots, H, d, dv) fp32
     is read (unless a sequence starts at position 0) and left at the step's last token. Returns o (T, H * dv).
     ``chunked`` picks the prompt form (64-token chunks as matrix products) over the token-by-token scan; by default
     steps that bring 8 or more tokens per sequence on average take it. ``max_len`` (the most tokens any sequence
     brings; 0: unknown) lets the prompt form run its chunks side by side when a sequence has more than one. The
-    prompt form needs ``pos`` (T,) and rotates / scales the q and k columns of ``proj`` in place."""
+    prompt form needs ``pos`` (T,) and rotates / scales the q and k columns of ``proj`` in place. ``act``: an activation
+    on q, k and v as projected, ahead of the rotation and the scale (the prompt form applies it in place)."""
     T, ld = proj.shape
     B = seq_slot.numel()
     if tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or decay.numel() != H:
@@ -219,7 +226,8 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: tor
                                         _opt(inv_freq, "inv_freq", F32), _dev(seq_start, "seq_start", I32),
                                         _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32),
                                         out.data_ptr(), B, H, d, dv, rot_dims, float(k_scale), int(bool(chunked)),
-                                        _opt(ws, "ws", F32), max_chunks, T, _opt(pos, "pos", I32), _stream()))
+                                        _opt(ws, "ws", F32), max_chunks, T, _opt(pos, "pos", I32), int(act),
+                                        _stream()))
     return out
 
 
@@ -325,20 +333,62 @@ def moe_route(proj: torch.Tensor, z_off: int, E: int, top: int):
     return ids, wts
 
 
-def moe_route_scores(proj: torch.Tensor, z_off: int, E: int, top: int, bias: Optional[torch.Tensor] = None):
-    """Softmax over all E router outputs at proj[:, z_off:]; the ``top`` largest of score + ``bias`` are chosen
-    (lowest index first among equals); the weights are the chosen scores themselves, not renormalised."""
+def moe_route_scores(proj: torch.Tensor, z_off: int, E: int, top: int, bias: Optional[torch.Tensor] = None,
+                     sigmoid: bool = False, square: bool = False):
+    """Softmax over all E router outputs at proj[:, z_off:] (``sigmoid``: the sigmoid of every output on its own); the
+    ``top`` largest of score + ``bias`` are chosen (lowest index first among equals); the weights are the chosen scores
+    themselves, not renormalised (``square``: their squares)."""
     T, ld = proj.shape
     if z_off + E > ld or (bias is not None and bias.numel() != E):
         raise ValueError("moe_route_scores: router logits outside the row, or the correction's size")
     ids = torch.empty(T, top, dtype=I32, device=proj.device)
     wts = torch.empty(T, top, dtype=F32, device=proj.device)
     _check(load_library().lgs_moe_route_scores(_dev(proj, "proj", F32) + 4 * z_off, ld, T, E, top,
-                                               _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), _stream()))
+                                               _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), int(sigmoid),
+                                               int(square), _stream()))
     return ids, wts
 
 
-def moe_router(h: torch.Tensor, w: torch.Tensor, top: int, bias: Optional[torch.Tensor] = None):
+def act_rows(proj: torch.Tensor, off: int, n: int, act: int, gate_off: int = -1, bf16: bool = False) -> torch.Tensor:
+    """act(proj[:, off:off + n]), times sigmoid(proj[:, gate_off]) row by row when ``gate_off`` >= 0; ``bf16``: rounded
+    to bf16 (a bf16 product's operand)."""
+    T, ld = proj.shape
+    if off + n > ld or gate_off >= ld:
+        raise ValueError("act_rows: columns outside the row")
+    out = torch.empty(T, n, dtype=torch.bfloat16 if bf16 else F32, device=proj.device)
+    base = _dev(proj, "proj", F32)
+    _check(load_library().lgs_act_rows(base + 4 * off, ld, base + 4 * gate_off if gate_off >= 0 else None, ld,
+                                       out.data_ptr(), int(bf16), T, n, act, _stream()))
+    return out
+
+
+def sandwich_step(x: torch.Tensor, *, branches=(), coef: float = 1.0, post_w: Optional[torch.Tensor] = None,
+                  next_w: Optional[torch.Tensor] = None, eps: float, want_f32: bool = True, bf16_copy: bool = False):
+    """One boundary between sublayers that are normed on the way in and out, in place on the residual x (T, W).
+    ``branches``: up to two (y, w) pairs of the sublayer that ran, each y (T, W) RMS-normed with weight w (w None: taken
+    as it is); their sum times ``coef`` is RMS-normed with ``post_w`` (the output norm's weight times the layer's
+    per-channel scale) and added to x. With ``next_w`` the next sublayer's input rmsnorm(x) * next_w is returned as
+    (h fp32 or None, h bf16 or None)."""
+    T, W = x.shape
+    ys = [(None, None), (None, None)]
+    for i, (y, w) in enumerate(branches):
+        if i > 1 or y.shape != (T, W) or (w is not None and w.numel() != W):
+            raise ValueError("sandwich_step: at most two branches of the residual's shape")
+        ys[i] = (y, w)
+    if (ys[0][0] is not None and (post_w is None or post_w.numel() != W)) or (next_w is not None and next_w.numel() != W):
+        raise ValueError("sandwich_step: norm weights")
+    h = torch.empty(T, W, dtype=F32, device=x.device) if next_w is not None and (want_f32 or not bf16_copy) else None
+    h16 = torch.empty(T, W, dtype=torch.bfloat16, device=x.device) if next_w is not None and bf16_copy else None
+    _check(load_library().lgs_sandwich_step(_dev(x, "x", F32), _opt(ys[0][0], "y0", F32), _opt(ys[0][1], "w0", F32),
+                                            _opt(ys[1][0], "y1", F32), _opt(ys[1][1], "w1", F32), float(coef),
+                                            _opt(post_w, "post_w", F32), _opt(next_w, "next_w", F32),
+                                            _opt(h, "h", F32), _opt(h16, "h_bf16", torch.bfloat16), float(eps), T, W,
+                                            _stream()))
+    return h, h16
+
+
+def moe_router(h: torch.Tensor, w: torch.Tensor, top: int, bias: Optional[torch.Tensor] = None, sigmoid: bool = False,
+               square: bool = False):
     """``moe_route_scores`` of the router logits w h, both in one launch (steps with few tokens). w (E, K)."""
     T, K = h.shape
     E = w.shape[0]
@@ -347,7 +397,8 @@ def moe_router(h: torch.Tensor, w: torch.Tensor, top: int, bias: Optional[torch.
     ids = torch.empty(T, top, dtype=I32, device=h.device)
     wts = torch.empty(T, top, dtype=F32, device=h.device)
     _check(load_library().lgs_moe_router(_dev(h, "h", F32), K, _dev(w, "w"), _wf32(w, "w"), T, K, E, top,
-                                         _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), _stream()))
+                                         _opt(bias, "bias", F32), ids.data_ptr(), wts.data_ptr(), int(sigmoid),
+                                         int(square), _stream()))
     return ids, wts
 
 
@@ -627,9 +678,13 @@ def softcap(z: torch.Tensor, cap: float) -> torch.Tensor:
 
 def normattn_prepare(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, cache_k: torch.Tensor,
                      cache_v: torch.Tensor, slot: torch.Tensor, pos: torch.Tensor, *, H: int, G: int, d: int, dv: int,
-                     eps: float, temp_coef: float = 0.0, temp_every: int = 0) -> None:
-    """Unit-RMS queries (times the position's query temperature) in place in ``proj``; unit-RMS keys and the values
-    into the cache rows (slot, position). cache_k (slots, S, G, d), cache_v (slots, S, G, dv)."""
+                     eps: float, temp_coef: float = 0.0, temp_every: int = 0, norm: bool = True,
+                     q_weight: Optional[torch.Tensor] = None, k_weight: Optional[torch.Tensor] = None,
+                     inv_freq: Optional[torch.Tensor] = None, rot_dims: int = 0) -> None:
+    """Queries normed (``norm``: divided by their root mean square, times ``q_weight`` (d,) if given), rotated on the
+    pairs (i, i + rot_dims / 2) and multiplied by the position's query temperature, in place in ``proj``; keys normed
+    (``k_weight``) and rotated alike, and the values, into the cache rows (slot, position). cache_k (slots, S, G, d),
+    cache_v (slots, S, G, dv). ``v_off == k_off`` (with dv == d): the values are the keys as projected."""
     T, ld = proj.shape
     slots, S = cache_k.shape[:2]
     if tuple(cache_k.shape) != (slots, S, G, d) or tuple(cache_v.shape) != (slots, S, G, dv) or \
@@ -637,28 +692,35 @@ def normattn_prepare(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, cac
         raise ValueError("normattn_prepare: cache shapes")
     if slot.numel() != T or pos.numel() != T:
         raise ValueError("normattn_prepare: one slot and position per row")
+    if any(w is not None and w.numel() != d for w in (q_weight, k_weight)) or rot_dims % 2 or rot_dims > d or \
+            (rot_dims > 0 and (inv_freq is None or inv_freq.numel() < rot_dims // 2)):
+        raise ValueError("normattn_prepare: norm weights of d values, rotary frequencies for rot_dims / 2 pairs")
     _check(load_library().lgs_normattn_prepare(_dev(proj, "proj", F32), ld, q_off, k_off, v_off,
                                                _dev(cache_k, "cache_k"), _dev(cache_v, "cache_v"),
                                                _wf32(cache_k, "cache_k"), _dev(slot, "slot", I32),
                                                _dev(pos, "pos", I32), T, H, G, d, dv, S, float(eps), float(temp_coef),
-                                               int(temp_every), _stream()))
+                                               int(temp_every), int(norm), _opt(q_weight, "q_weight", F32),
+                                               _opt(k_weight, "k_weight", F32), _opt(inv_freq, "inv_freq", F32),
+                                               int(rot_dims), _stream()))
 
 
 def sinkattn(proj: torch.Tensor, q_off: int, cache_k: torch.Tensor, cache_v: torch.Tensor,
              sink: Optional[torch.Tensor], seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor,
              max_len: int, *, H: int, G: int, d: int, dv: int, scale: float, chunk: int = 0, cap: float = 0.0,
-             post: float = 1.0, bf16_copy: bool = False, splits: Optional[int] = None) -> torch.Tensor:
+             post: float = 1.0, bf16_copy: bool = False, splits: Optional[int] = None,
+             gate_off: int = -1) -> torch.Tensor:
     """Causal softmax attention of every row of a packed batch over its sequence's cached keys and values, grouped
     key / value heads, with exp(sink[h]) in the normaliser; the prepared queries are the H d columns of ``proj`` at
-    ``q_off``. Returns (T, H dv) fp32 times ``post``, or with ``bf16_copy`` its rounding to bf16."""
+    ``q_off``. ``gate_off`` >= 0: head h's output is multiplied by sigmoid(proj[:, gate_off + h]). Returns (T, H dv)
+    fp32 times ``post``, or with ``bf16_copy`` its rounding to bf16."""
     T, ld = proj.shape
     B = seq_slot.numel()
     slots, S = cache_k.shape[:2]
     if tuple(cache_k.shape) != (slots, S, G, d) or tuple(cache_v.shape) != (slots, S, G, dv):
         raise ValueError("sinkattn: cache shapes")
     if seq_start.numel() != B + 1 or q_off + H * d > ld or not 1 <= max_len <= T or \
-            (sink is not None and sink.numel() != H):
-        raise ValueError("sinkattn: step table / query columns / sink")
+            (sink is not None and sink.numel() != H) or gate_off + H > ld:
+        raise ValueError("sinkattn: step table / query columns / sink / head gates")
     out = torch.empty(T, H * dv, dtype=F32, device=proj.device)
     out16 = torch.empty(T, H * dv, dtype=torch.bfloat16, device=proj.device) if bf16_copy else None
     if max_len > 1:
@@ -673,14 +735,18 @@ def sinkattn(proj: torch.Tensor, q_off: int, cache_k: torch.Tensor, cache_v: tor
                                        _dev(seq_pos0, "seq_pos0", I32), out.data_ptr(),
                                        _opt(out16, "out_bf16", torch.bfloat16), _opt(part, "part", F32), splits, B,
                                        int(max_len), H, G, d, dv, S, int(chunk), float(scale), float(cap), float(post),
+                                       _dev(proj, "proj", F32) + 4 * gate_off if gate_off >= 0 else None, ld,
                                        _stream()))
     return out16 if bf16_copy else out
 
 
 def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tensor, b_off: int, A_log: torch.Tensor,
                   dt_bias: torch.Tensor, *, H: int, G: int, d: int, per_channel: bool, q_scale: float,
-                  norm_eps: float = 1e-6, w_a2: Optional[torch.Tensor] = None):
-    """qkv (T, 2 G d + H dv): q and k become unit vectors per head in place (q also times ``q_scale``). The raw decay
+                  norm_eps: float = 1e-6, w_a2: Optional[torch.Tensor] = None, unit: bool = True,
+                  decay_form: int = 0, tau: float = 1.0, qkv_off: int = 0):
+    """qkv (T, ld) holds q | k (G d each) from column ``qkv_off``. ``unit``: q and k become unit vectors per head in
+    place (q also times ``q_scale``); otherwise q is only scaled. ``decay_form`` 1: the decays are
+    sigmoid(a + dt_bias)^(1 / tau) (``A_log`` None). ``b`` None: no betas. The raw decay
     inputs are the H d (``per_channel``) or H columns of ``a`` at ``a_off`` - or, with ``w_a2`` (H d or H, rank), w_a2
     times the rank columns there; the raw betas are the H columns of ``b`` at ``b_off``. Returns (dec, beta, kq):
     exp(-exp(A_log) softplus(a + dt_bias)) (T, H d) or (T, H), sigmoid(b) (T, H), and k . q of the prepared vectors
@@ -688,18 +754,21 @@ def delta_prepare(qkv: torch.Tensor, a: torch.Tensor, a_off: int, b: torch.Tenso
     T, ld = qkv.shape
     n = H * d if per_channel else H
     cols = n if w_a2 is None else w_a2.shape[1]
-    if a.shape[0] != T or b.shape[0] != T or a_off + cols > a.shape[1] or b_off + H > b.shape[1] or \
-            A_log.numel() != H or dt_bias.numel() != n or ld < 2 * G * d or (w_a2 is not None and w_a2.shape[0] != n):
+    if a.shape[0] != T or a_off + cols > a.shape[1] or (b is not None and (b.shape[0] != T or b_off + H > b.shape[1])) or \
+            (decay_form == 0 and (A_log is None or A_log.numel() != H)) or dt_bias.numel() != n or \
+            ld < qkv_off + 2 * G * d or (w_a2 is not None and w_a2.shape[0] != n) or decay_form not in (0, 1):
         raise ValueError("delta_prepare: shapes")
     dec = torch.empty(T, n, dtype=F32, device=qkv.device)
-    beta = torch.empty(T, H, dtype=F32, device=qkv.device)
+    beta = torch.empty(T, H, dtype=F32, device=qkv.device) if b is not None else None
     kq = torch.empty(T, G, dtype=F32, device=qkv.device)
-    _check(load_library().lgs_delta_prepare(_dev(qkv, "qkv", F32), ld, _dev(a, "a", F32) + 4 * a_off, a.shape[1],
-                                            _dev(b, "b", F32) + 4 * b_off, b.shape[1], _dev(A_log, "A_log", F32),
-                                            _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), beta.data_ptr(),
+    _check(load_library().lgs_delta_prepare(_dev(qkv, "qkv", F32) + 4 * qkv_off, ld, _dev(a, "a", F32) + 4 * a_off,
+                                            a.shape[1], _dev(b, "b", F32) + 4 * b_off if b is not None else None,
+                                            b.shape[1] if b is not None else 0, _opt(A_log, "A_log", F32),
+                                            _dev(dt_bias, "dt_bias", F32), dec.data_ptr(), _opt(beta, "beta", F32),
                                             kq.data_ptr(), T, H, G, d, int(per_channel), float(q_scale),
                                             float(norm_eps), _opt(w_a2, "w_a2"), 0 if w_a2 is None else w_a2.shape[1],
-                                            0 if w_a2 is None else _wf32(w_a2, "w_a2"), _stream()))
+                                            0 if w_a2 is None else _wf32(w_a2, "w_a2"), int(unit), int(decay_form),
+                                            float(tau), _stream()))
     return dec, beta, kq
 
 
@@ -734,21 +803,27 @@ def delta_step_prepare(proj: torch.Tensor, off: int, conv_w: torch.Tensor, conv_
     return qkv, dec, beta, kq
 
 
-def gated_delta(qkv: torch.Tensor, dec: torch.Tensor, beta: torch.Tensor, kq: torch.Tensor, state: torch.Tensor,
-                seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor, *, H: int, G: int, d: int,
-                dv: int, per_channel: bool, lanes: int = 0) -> torch.Tensor:
+def gated_delta(qkv: torch.Tensor, dec: torch.Tensor, beta: Optional[torch.Tensor], kq: torch.Tensor,
+                state: torch.Tensor, seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor, *, H: int,
+                G: int, d: int, dv: int, per_channel: bool, lanes: int = 0, plain: bool = False,
+                qkv_off: int = 0) -> torch.Tensor:
     """The gated delta rule over a packed batch, token by token: S <- diag(dec) S; u = beta (v - S^T k);
     S <- S + k u^T; o = S^T q. qkv (T, 2 G d + H dv) prepared rows, kq (T, G) their k . q (``delta_prepare``); state
     (slots, H, d, dv) fp32 is read unless a sequence starts at position 0 and left at the step's last token. Returns
-    o (T, H dv). ``lanes``: lanes that share one state column (4, 8, 16; 0: chosen from the sizes)."""
+    o (T, H dv). ``lanes``: lanes that share one state column (4, 8, 16; 0: chosen from the sizes). ``plain``: the
+    rule without the correction, S <- diag(dec) S + k v^T, o = S^T q (``beta`` None). ``qkv_off``: the first column of
+    q | k | v in wider rows."""
     T, ld = qkv.shape
     B = seq_slot.numel()
-    if ld != 2 * G * d + H * dv or tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or \
-            dec.shape != (T, H * d if per_channel else H) or beta.shape != (T, H) or kq.shape != (T, G):
+    if ld < qkv_off + 2 * G * d + H * dv or tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or \
+            dec.shape != (T, H * d if per_channel else H) or (not plain and (beta is None or beta.shape != (T, H))) or \
+            kq.shape != (T, G):
         raise ValueError("gated_delta: shapes")
     out = torch.empty(T, H * dv, dtype=F32, device=qkv.device)
-    _check(load_library().lgs_gated_delta(_dev(qkv, "qkv", F32), ld, _dev(dec, "dec", F32), _dev(beta, "beta", F32),
+    _check(load_library().lgs_gated_delta(_dev(qkv, "qkv", F32) + 4 * qkv_off, ld, _dev(dec, "dec", F32),
+                                          _opt(beta, "beta", F32) if plain else _dev(beta, "beta", F32),
                                           _dev(kq, "kq", F32), _dev(state, "state", F32), _dev(seq_start, "seq_start", I32),
                                           _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32),
-                                          out.data_ptr(), B, H, G, d, dv, int(per_channel), int(lanes), _stream()))
+                                          out.data_ptr(), B, H, G, d, dv, int(per_channel), int(lanes), int(plain),
+                                          _stream()))
     return out
