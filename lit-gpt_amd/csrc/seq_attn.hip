@@ -114,21 +114,20 @@ __global__ void __launch_bounds__(256) normattn_prepare_kernel(NormPrepArgs p) {
     const bool isk = vec >= p.H;
     float* x = row + (isk ? p.k_off + (size_t)(vec - p.H) * d : p.q_off + (size_t)vec * d);
     const float* w = isk ? p.k_w : p.q_w;
-    float s = 1.0f;
+    float s = isk ? 1.0f : temp;  // the norm's factor and the query temperature as one number
     if (p.norm) {
       float ss = 0.0f;
       for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
       ss = wave_sum(ss);
-      s = 1.0f / sqrtf(ss / (float)d + p.eps);
+      s = s / sqrtf(ss / (float)d + p.eps);
     }
-    const float post = isk ? 1.0f : temp;
     const size_t kat = (crow + (vec - p.H)) * d;
     for (int i = lane; i < half; i += 64) {  // a lane owns both members of a rotated pair
       float u = x[i] * s, v = x[i + half] * s;
       if (w) u *= w[i], v *= w[i + half];
       float sn, cs;
       sincosf(fpos * p.inv_freq[i], &sn, &cs);
-      const float a = (u * cs - v * sn) * post, b = (v * cs + u * sn) * post;
+      const float a = u * cs - v * sn, b = v * cs + u * sn;
       if (isk) {
         cstore<CF32>(p.cache_k, kat + i, a);
         cstore<CF32>(p.cache_k, kat + i + half, b);
@@ -141,7 +140,7 @@ __global__ void __launch_bounds__(256) normattn_prepare_kernel(NormPrepArgs p) {
       float u = x[i] * s;
       if (w) u *= w[i];
       if (isk) cstore<CF32>(p.cache_k, kat + i, u);
-      else x[i] = u * post;
+      else x[i] = u;
     }
   }
   __syncthreads();

@@ -303,11 +303,12 @@ def _mixer_shapes(p: str, m, W: int) -> Dict[str, Tuple[int, ...]]:
             out.update({p + "left.out": (W,), p + "right.out": (W,)})
         return out
     if m.kind in ("sink_attention", "rotary_attention", "key_value_attention"):
-        out = {p + "q": (m.heads * m.dim, W), p + "k": (m.kv_heads * m.dim, W), p + "o": (W, m.heads * m.vdim)}
+        out = {p + "q": (m.heads * m.dim, W), p + "k": (m.kv_heads * m.dim, W)}
         if m.values == "own":
             out[p + "v"] = (m.kv_heads * m.vdim, W)
         if m.sink_kind == "learned":
             out[p + "sink"] = (m.heads,)
+        out[p + "o"] = (W, m.heads * m.vdim)
         if m.qk_norm == "weight":
             out.update({p + "q.norm": (m.dim,), p + "k.norm": (m.dim,)})
         if m.head_gate:
