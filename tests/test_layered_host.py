@@ -360,3 +360,130 @@ def test_ravelorn_plain_implementation():
     rw = {"router": torch.tensor([[0.0, 0.0], [9.0, 9.0]], dtype=torch.float64)}
     out = orc.moe_ff(h, rw, {"router": {"experts": 0, "identity": 2, "top": 1}})
     assert torch.allclose(out, torch.softmax(torch.tensor([0.0, 18.0], dtype=torch.float64), 0)[1] * h)
+
+
+# ------------------------------------------------------------------------------------------------ the Gatutar design
+def _gat_cfg():
+    return {
+        "architecture": "Gatutar", "vocab": 23, "width": 16, "norm": {"eps": 1e-5},
+        "layers": [
+            {"type": "parallel_2", "mlp": {"kind": "dense", "ff": 10},
+             "mixer": {"left": {"heads": 4, "kv_heads": 2, "dim": 6, "vdim": 6, "scale": 0.3, "q_temp": {"coef": 0.5, "every": 4}},
+                       "right": {"heads": 2, "dim": 5, "vdim": 3, "decay": [0.5, 0.9]}}},
+            {"type": "parallel", "mlp": {"kind": "moe", "expert": {"ff": 6}, "router": {"experts": 3, "top": 2},
+                                         "shared": {"ff": 4}},
+             "mixer": {"left": {"heads": 6, "kv_heads": 3, "dim": 4, "vdim": 2, "scale": 0.5,
+                                "rot": {"dims": 2, "base": 100.0,
+                                        "scaling": {"factor": 2.0, "low": 1.0, "high": 4.0, "original": 16}}},
+                       "right": {"heads": 2, "dim": 3, "vdim": 5, "tau": 3.0}}},
+            {"type": "parallel", "mlp": None,
+             "mixer": {"left": {"heads": 1, "kv_heads": 1, "dim": 4, "vdim": 4, "scale": 0.5},
+                       "right": {"heads": 1, "dim": 2, "vdim": 2, "tau": 1.0}}},
+        ],
+    }
+
+
+def test_gatutar_config_and_tensor_names():
+    from lit_gpt.config import LayeredConfig, model_class
+    from lit_gpt.layered import LayeredGPT
+
+    c = LayeredConfig.from_dict(_gat_cfg())
+    assert model_class(c) is LayeredGPT
+    d = c.design
+    assert (d.block, d.norm, d.dense_ff, d.moe, d.tied_head, d.norm_offset) == ("sandwich", "rms", "relu2", "sigmoid", False, 0.0)
+    a, b, e = (l.mixer for l in c.layers)
+    assert (a.kind, a.branch_norm, a.left_scale, a.right_scale) == ("parallel", True, 0.5, 0.5)
+    assert (a.left.kind, a.left.heads, a.left.kv_heads, a.left.qk_norm, a.left.sink_kind, a.left.values, a.left.head_gate,
+            a.left.q_temp_coef, a.left.q_temp_every, a.left.rot.dims) == \
+        ("key_value_attention", 4, 2, "weight", "none", "keys", True, 0.5, 4, 0)
+    assert (a.right.kind, a.right.decay, a.right.dim, a.right.vdim) == ("lightning", [0.5, 0.9], 5, 3)
+    assert (b.left.kind, b.left.qk_norm, b.left.sink_kind, b.left.values, b.left.head_gate, b.left.rot.dims) == \
+        ("rotary_attention", "none", "one", "own", False, 2)
+    assert b.left.rot.scaling == {"factor": 2.0, "low": 1.0, "high": 4.0, "original": 16.0}
+    assert (b.right.kind, b.right.tau) == ("gated_linear", 3.0) and e.left.rot.dims == 0
+    f = c.layers[1].mlp
+    assert (f.experts, f.top, f.ff, f.shared_ff) == (3, 2, 6, 4) and c.layers[2].mlp is None
+    assert c.layers[0].mlp.kind == "dense" and c.layers[0].mlp.ff == 10
+    shapes = LayeredGPT.tensor_shapes(c)
+    assert shapes["head"] == (23, 16) and shapes["final.norm"] == (16,) and "pos" not in shapes
+    for n in ("norm1", "norm1b", "norm2", "norm2b", "ls1", "ls2"):
+        assert shapes[f"l0.{n}"] == (16,)
+    assert "l2.norm2" not in shapes and "l2.ls2" not in shapes and shapes["l2.ls1"] == (16,)
+    assert shapes["l0.mix.left.q"] == (24, 16) and shapes["l0.mix.left.k"] == (12, 16) and "l0.mix.left.v" not in shapes
+    assert shapes["l0.mix.left.q.norm"] == (6,) and shapes["l0.mix.left.g"] == (4, 16) and shapes["l0.mix.left.o"] == (16, 24)
+    assert shapes["l0.mix.right.q"] == (10, 16) and shapes["l0.mix.right.v"] == (6, 16) and shapes["l0.mix.right.norm"] == (6,)
+    assert shapes["l0.mix.left.out"] == (16,) and shapes["l0.mix.right.out"] == (16,)
+    assert shapes["l0.mlp.up"] == (10, 16) and "l0.mlp.gate" not in shapes
+    assert shapes["l1.mix.left.v"] == (6, 16) and shapes["l1.mix.left.o"] == (16, 12) and "l1.mix.left.sink" not in shapes
+    assert shapes["l1.mix.right.a2"] == (6, 16) and shapes["l1.mix.right.a2.b"] == (6,) and shapes["l1.mix.right.norm"] == (5,)
+    assert shapes["l1.mlp.router"] == (3, 16) and shapes["l1.mlp.e2.up"] == (6, 16) and "l1.mlp.e2.gate" not in shapes
+    assert shapes["l1.mlp.shared.up"] == (4, 16) and shapes["l1.mlp.shared.sg"] == (1, 16)
+    w = LayeredGPT.random_weights(c)
+    assert set(w) == set(shapes) and all(tuple(w[k].shape) == shapes[k] for k in shapes)
+
+
+@pytest.mark.parametrize("edit", [
+    lambda c: c["layers"][0]["mixer"]["left"].update(kv_heads=3),  # heads no multiple of the key heads
+    lambda c: c["layers"][0]["mixer"]["left"].update(vdim=5),  # values that are the keys have the keys' size
+    lambda c: c["layers"][0]["mixer"]["right"].update(decay=[0.5]),  # one decay per head
+    lambda c: c["layers"][1]["mixer"]["left"]["rot"].update(dims=6),  # more rotary dims than the head has
+    lambda c: c["layers"][1]["mixer"]["left"]["rot"].update(dims=3),
+    lambda c: c["layers"][1]["mixer"]["right"].update(tau=0.0),
+    lambda c: c["layers"][1]["mixer"]["right"].update(dim=600),
+    lambda c: c["layers"][1]["mlp"]["router"].update(top=4),
+])
+def test_gatutar_config_rejects_what_does_not_fit(edit):
+    from lit_gpt.config import LayeredConfig
+
+    c = _gat_cfg()
+    edit(c)
+    with pytest.raises(ValueError):
+        LayeredConfig.from_dict(c)
+
+
+def test_gatutar_plain_implementation():
+    import math
+
+    from lit_gpt.config import LayeredConfig, RotarySpec
+    from lit_gpt.layered import LayeredGPT
+    from oracle import gatutar as orc
+
+    cfg = _gat_cfg()
+    w = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=3)
+    toks = [3, 7, 1, 0, 22, 5, 9, 9, 4, 13, 2, 8]
+    full = orc.forward(cfg, w, toks)
+    assert torch.allclose(orc.forward(cfg, w, toks[:7]), full[:7], atol=1e-10)  # causal
+    D = torch.float64
+    eye = torch.eye(2, dtype=D)
+    h = torch.tensor([[1.0, 1.0]], dtype=D)
+    # one key whose score is 0: with the extra one in the denominator the weight is a half
+    m = {"heads": 1, "kv_heads": 1, "dim": 2, "vdim": 2, "scale": 0.0}
+    out = orc.rope_attention(h, m, {"q": eye, "k": eye, "v": eye, "o": eye})
+    assert torch.allclose(out, 0.5 * h)
+    # a rotation by position p turns the pair (1, 0) by the angle p * f; dims beyond the rotated ones pass
+    r = orc.rotate_half(torch.tensor([1.0, 5.0, 0.0, 7.0], dtype=D)[[0, 2, 1, 3]], 3, [0.25])  # pairs (0, 1) of a 2-dim rotation
+    assert torch.allclose(r, torch.tensor([math.cos(0.75), math.sin(0.75), 5.0, 7.0], dtype=D))
+    # frequency bands: short waves kept, long ones divided by the factor, the same numbers as the product's table
+    rot = {"dims": 8, "base": 100.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 40}}
+    f = orc.scaled_frequencies(rot)
+    assert f[0] == 1.0 and f[-1] == pytest.approx(100.0 ** -0.75 / 4.0)
+    assert f == pytest.approx(RotarySpec(8, 100.0, rot["scaling"]).inv_freq(), rel=1e-12)
+    # the linear rule: without decay the state is the sum of the outer products
+    q = torch.tensor([[[1.0, 0.0]], [[0.0, 1.0]]], dtype=D)
+    k = torch.tensor([[[1.0, 0.0]], [[1.0, 1.0]]], dtype=D)
+    v = torch.tensor([[[2.0]], [[3.0]]], dtype=D)
+    o = orc.linear_recurrence(q, k, v, torch.ones(2, 1, 2, dtype=D))
+    assert o.view(-1).tolist() == [2.0, 3.0]
+    o = orc.linear_recurrence(q.flip(0), k, v, torch.full((2, 1, 2), 0.5, dtype=D))
+    assert o.view(-1).tolist() == [0.0, 0.5 * 2.0 + 3.0]
+    # the router's score scales the expert's input: with relu^2 experts the output goes with its square
+    fw = {"router": torch.tensor([[0.0, 0.0], [1.0, 1.0]], dtype=D), "e0.up": eye, "e0.down": eye, "e1.up": eye, "e1.down": eye}
+    out = orc.feed_forward(h, {"kind": "moe", "router": {"experts": 2, "top": 1}}, fw)
+    assert torch.allclose(out, torch.sigmoid(torch.tensor(2.0, dtype=D)) ** 2 * h)
+    # a shut shared gate leaves the routed experts alone; an open one adds the shared expert
+    fs = dict(fw, **{"shared.up": eye, "shared.down": eye, "shared.sg": torch.tensor([[-50.0, 0.0]], dtype=D)})
+    shut = orc.feed_forward(h, {"kind": "moe", "router": {"experts": 2, "top": 1}, "shared": {"ff": 2}}, fs)
+    assert torch.allclose(shut, out)
+    fs["shared.sg"] = torch.tensor([[50.0, 0.0]], dtype=D)
+    opened = orc.feed_forward(h, {"kind": "moe", "router": {"experts": 2, "top": 1}, "shared": {"ff": 2}}, fs)
+    assert torch.allclose(opened, out + h)
