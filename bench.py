@@ -721,6 +721,65 @@ def delta_bench(args) -> None:
         print(json.dumps(line), flush=True)
 
 
+def sandwich_bench(args) -> None:
+    """``--sandwich``: prefill and decode throughput of the Gatutar design (sandwich-normed layers whose mixers run a
+    softmax attention and a linear-attention rule side by side: key-value attention beside the constant-decay rule,
+    rotary attention with a sink of score 0 beside the gated linear attention; ungated relu^2 feed-forwards alternating
+    with sigmoid-routed experts plus a shared expert; random bf16 weights) at sizes that resemble a real model's
+    layers, beside the closest existing model of the framework - the Ravelorn layers of ``--delta`` (sink attention
+    beside a delta rule, delta-rule layers, score-routed gated experts) - at equal width, depth, head counts and
+    active feed-forward size. One JSON line per size: one 2048-token prompt (warm, median of 3) and captured greedy
+    decode steps at context 2048, for 1 and 8 sequences."""
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+
+    dev = torch.device("cuda", 0)
+    T, L, V = args.prompt_len, 4, 32000
+    sizes = {"w2048": (2048, 5632), "w4096": (4096, 11008)}
+    for name, (W, ff) in sizes.items():
+        if args.sandwich not in ("all", name):
+            continue
+        H = W // 128
+        E, top = 16, 4
+        moe = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": E, "top": top}, "shared": {"ff": ff // top}}
+        dense = {"kind": "dense", "ff": ff}
+        kv = {"type": "parallel_2", "mixer": {
+            "left": {"heads": H, "kv_heads": H // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "q_temp": {"coef": 0.1, "every": 512}},
+            "right": {"heads": H // 2, "dim": 128, "vdim": 128,
+                      "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(1, H // 2 - 1)) for i in range(H // 2)]}}}
+        rot = {"type": "parallel", "mixer": {
+            "left": {"heads": H, "kv_heads": H // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "rot": {"dims": 64, "base": 5e5, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+            "right": {"heads": H // 2, "dim": 128, "vdim": 128, "tau": 16.0, "decay_rank": W // 32}}}
+        cfg = LayeredConfig.from_dict({"architecture": "Gatutar", "vocab": V, "width": W, "norm": {"eps": 1e-5},
+                                       "layers": [dict(kv, mlp=dense), dict(rot, mlp=moe), dict(kv, mlp=dense),
+                                                  dict(rot, mlp=moe)]})
+        line = {"bench": "sandwich", "size": name, "width": W, "ff": ff, "layers": L, "prompt_len": T, "steps": args.steps,
+                "dtype": "bf16", "data": "synthetic"}
+        model = LayeredGPT(cfg, LayeredGPT.random_weights(cfg, seed=1), device=dev, dtype=torch.bfloat16)
+        line["gatutar"] = _layered_timings(model, args, T, V)
+        del model
+        torch.cuda.empty_cache()
+        ident = 2
+        rmoe = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": E, "identity": ident, "top": top}}
+        cd = {"type": "channel_delta", "mixer": {"heads": H, "kv_heads": H, "dim": 128, "vdim": 128, "conv": 4,
+                                                 "decay_rank": W // 32, "gate_rank": W // 32}, "mlp": rmoe}
+        par = {"type": "parallel", "mlp": rmoe, "mixer": {
+            "left": {"heads": H, "kv_heads": H // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "q_temp": {"coef": 0.1, "every": 512}},
+            "right": {"heads": H // 2, "kv_heads": H // 2, "dim": 128, "vdim": 128, "conv": 4},
+            "left_scale": 1.0, "right_scale": 1.0}}
+        rcfg = LayeredConfig.from_dict({"architecture": "Ravelorn", "vocab": V, "width": W, "norm": {"eps": 1e-5},
+                                        "residual_mult": 0.7, "logit_softcap": 30.0, "max_positions": 4096,
+                                        "layers": [cd, par, cd, par]})
+        model = LayeredGPT(rcfg, LayeredGPT.random_weights(rcfg, seed=1), device=dev, dtype=torch.bfloat16)
+        line["ravelorn_layers"] = _layered_timings(model, args, T, V)
+        del model
+        torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -733,6 +792,9 @@ def main():
     ap.add_argument("--delta", nargs="?", const="all", default=None, choices=("all", "w2048", "w4096"),
                     help="instead of the headline run: the Ravelorn design (gated delta rule, sink attention, routed "
                          "experts) beside the Rigulorn layers at equal size")
+    ap.add_argument("--sandwich", nargs="?", const="all", default=None, choices=("all", "w2048", "w4096"),
+                    help="instead of the headline run: the Gatutar design (sandwich norms, softmax attention beside "
+                         "linear-attention rules, sigmoid-routed experts) beside the Ravelorn layers at equal size")
     # defaults: the eager capture step (p = 2048) + 14 warm-up + 240 timed steps = the 255 decode steps of
     # SURVEY §8d (p = 2048 ... 2302)
     ap.add_argument("--steps", type=int, default=240)
@@ -758,6 +820,8 @@ def main():
         return hybrid_bench(args)
     if args.delta:
         return delta_bench(args)
+    if args.sandwich:
+        return sandwich_bench(args)
     traffic = {k: (None, "skipped") for k in ("gemv", "attention")}
     under_profiler = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
     headline = args.model == MODEL and args.quantize == "int4-g128"

@@ -62,32 +62,42 @@ __device__ __forceinline__ float decay_of(const DeltaPrepArgs& p, float z, int h
 // unit vectors; all threads walk the decays and betas; then k . q per key head.
 constexpr int kMaxRank = 512;  // inner size of a low-rank second map that is folded into a consuming kernel
 
+// part 0 of a row's work: the vectors (wave w takes the vectors w, w + 4, ...), the betas and k . q per key head;
+// part y >= 1: the decays [256 (y - 1), 256 y) - with `whole` (one workgroup per row) all of them
 template <bool A2F32>
-__device__ __forceinline__ void delta_prepare_row(const DeltaPrepArgs& p, size_t t) {
+__device__ __forceinline__ void delta_prepare_row(const DeltaPrepArgs& p, size_t t, int part, bool whole) {
   __shared__ float a1[kMaxRank];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int d = p.d;
   float* row = p.qkv + t * p.ld;
-  if (p.w_a2)
-    for (int r = threadIdx.x; r < p.rank; r += 256) a1[r] = aop<A2F32>(p.a[t * p.lda + r]);
-  __syncthreads();
+  if (part > 0 || whole) {
+    if (p.w_a2) {
+      for (int r = threadIdx.x; r < p.rank; r += 256) a1[r] = aop<A2F32>(p.a[t * p.lda + r]);
+      __syncthreads();
+    }
+    const int dc = p.per_channel ? d : 1, n = p.H * dc;
+    const int lo = whole ? 0 : 256 * (part - 1), hi = whole ? n : min(n, lo + 256);
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+      const float raw = p.w_a2 ? lowrank_dot<A2F32>(p.w_a2, i, a1, p.rank) : p.a[t * p.lda + i];
+      p.dec[t * n + i] = decay_of(p, raw + p.dt_bias[i], i / dc);
+    }
+    if (!whole) return;
+  }
   for (int vec = wave; vec < 2 * p.G; vec += 4) {
     float* x = row + (size_t)vec * d;
-    float ss = 0.0f;
-    for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
-    ss = wave_sum(ss);
-    const float s = p.unit ? (vec < p.G ? p.q_scale : 1.0f) / sqrtf(ss + p.norm_eps) : (vec < p.G ? p.q_scale : 1.0f);
+    float s = vec < p.G ? p.q_scale : 1.0f;
+    if (p.unit) {
+      float ss = 0.0f;
+      for (int i = lane; i < d; i += 64) ss = fmaf(x[i], x[i], ss);
+      ss = wave_sum(ss);
+      s = s / sqrtf(ss + p.norm_eps);
+    }
     if (s != 1.0f)
       for (int i = lane; i < d; i += 64) x[i] *= s;
   }
-  const int dc = p.per_channel ? d : 1, n = p.H * dc;
-  for (int i = threadIdx.x; i < n; i += 256) {
-    const float raw = p.w_a2 ? lowrank_dot<A2F32>(p.w_a2, i, a1, p.rank) : p.a[t * p.lda + i];
-    p.dec[t * n + i] = decay_of(p, raw + p.dt_bias[i], i / dc);
-  }
   if (p.b)
     for (int h = threadIdx.x; h < p.H; h += 256) p.beta[t * p.H + h] = sigmoid_f(p.b[t * p.ldb + h]);
-  __syncthreads();  // the unit vectors of all heads are written
+  __syncthreads();  // the prepared vectors of all heads are written
   for (int g = wave; g < p.G; g += 4) {
     const float *q = row + (size_t)g * d, *k = row + (size_t)(p.G + g) * d;
     float s = 0.0f;
@@ -97,10 +107,10 @@ __device__ __forceinline__ void delta_prepare_row(const DeltaPrepArgs& p, size_t
   }
 }
 
-// grid (T)
+// grid (T), or for steps of few rows (T, 1 + ceil(n / 256)): the decays in workgroups of their own
 template <bool A2F32>
 __global__ void __launch_bounds__(256) delta_prepare_kernel(DeltaPrepArgs p) {
-  delta_prepare_row<A2F32>(p, blockIdx.x);
+  delta_prepare_row<A2F32>(p, blockIdx.x, blockIdx.y, gridDim.y == 1);
 }
 
 // One channel of the short convolution for a one-token step: the weighted sum of the token's input and the slot's
@@ -386,8 +396,11 @@ extern "C" int lgs_delta_prepare(float* qkv, long ld, const float* a, long lda, 
   lgs::DeltaPrepArgs p{qkv, ld, a, lda, b, ldb, A_log, dt_bias, dec, beta, kq, H, G, d, per_channel ? 1 : 0, q_scale,
                        norm_eps, w_a2, rank, a2_f32, unit ? 1 : 0, decay_form, tau, nullptr, 0, nullptr, 0, 0, 0, nullptr,
                        nullptr, nullptr};
-  if (a2_f32) lgs::delta_prepare_kernel<true><<<T, 256, 0, stream>>>(p);
-  else lgs::delta_prepare_kernel<false><<<T, 256, 0, stream>>>(p);
+  // few rows (decode): the decays - with a low-rank second map a product each - spread over workgroups of their own
+  const int n = per_channel ? H * d : H;
+  const dim3 grid(T, T <= 64 && n > 256 ? 1 + (n + 255) / 256 : 1);
+  if (a2_f32) lgs::delta_prepare_kernel<true><<<grid, 256, 0, stream>>>(p);
+  else lgs::delta_prepare_kernel<false><<<grid, 256, 0, stream>>>(p);
   LGA_LAUNCH_RETURN();
 }
 

@@ -202,25 +202,47 @@ struct SandwichArgs {
   int n;
 };
 
+// sums of two values over the 256 threads of a workgroup in one round (`red` holds 8 floats)
+__device__ __forceinline__ void block_sum2_256(float& u, float& v, float* red) {
+  u = wave_sum(u);
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    red[threadIdx.x >> 6] = u;
+    red[4 + (threadIdx.x >> 6)] = v;
+  }
+  __syncthreads();
+  u = (red[0] + red[1]) + (red[2] + red[3]);
+  v = (red[4] + red[5]) + (red[6] + red[7]);
+}
+
 template <int CPT>
 __global__ void __launch_bounds__(256) sandwich_step_kernel(SandwichArgs p) {
-  __shared__ float red[4];
+  __shared__ float red[8];
   const size_t r = blockIdx.x;
   const int n = p.n, tid = threadIdx.x;
   float* xr = p.x + r * n;
   const float inv_n = 1.0f / (float)n;
-  float xv[CPT];
+  // every operand of the registers' share of the row is fetched up front, so that the reductions below wait for
+  // one round of loads only
+  float xv[CPT], av[CPT], bv[CPT], w0[CPT], w1[CPT], wp[CPT], wn[CPT];
+  const float *a = p.y0 ? p.y0 + r * n : nullptr, *b = p.y1 ? p.y1 + r * n : nullptr;
 #pragma unroll
-  for (int e = 0; e < CPT; ++e) xv[e] = tid + 256 * e < n ? xr[tid + 256 * e] : 0.0f;
-  if (p.y0) {
-    const float *a = p.y0 + r * n, *b = p.y1 ? p.y1 + r * n : nullptr;
-    float av[CPT], bv[CPT];
+  for (int e = 0; e < CPT; ++e) {
+    const int i = tid + 256 * e;
+    const bool in = i < n;
+    xv[e] = in ? xr[i] : 0.0f;
+    av[e] = (a && in) ? a[i] : 0.0f;
+    bv[e] = (b && in) ? b[i] : 0.0f;
+    w0[e] = (a && p.w0 && in) ? p.w0[i] : 1.0f;
+    w1[e] = (b && p.w1 && in) ? p.w1[i] : 1.0f;
+    wp[e] = (a && in) ? p.post_w[i] : 0.0f;
+    wn[e] = (p.next_w && in) ? p.next_w[i] : 0.0f;
+  }
+  if (a) {
     float sa = 0.0f, sb = 0.0f;
 #pragma unroll
     for (int e = 0; e < CPT; ++e) {
-      const int i = tid + 256 * e;
-      av[e] = i < n ? a[i] : 0.0f;
-      bv[e] = (b && i < n) ? b[i] : 0.0f;
       sa = fmaf(av[e], av[e], sa);
       sb = fmaf(bv[e], bv[e], sb);
     }
@@ -229,22 +251,27 @@ __global__ void __launch_bounds__(256) sandwich_step_kernel(SandwichArgs p) {
       if (b) sb = fmaf(b[i], b[i], sb);
     }
     float ra = 1.0f, rb = 1.0f;
-    if (p.w0) ra = 1.0f / sqrtf(block_sum_256(sa, red) * inv_n + p.eps);
-    if (b && p.w1) rb = 1.0f / sqrtf(block_sum_256(sb, red) * inv_n + p.eps);
-    auto joined = [&](int i, float ya, float yb) {
-      float s = p.w0 ? ya * ra * p.w0[i] : ya;
-      if (b) s += p.w1 ? yb * rb * p.w1[i] : yb;
+    if (p.w0 || (b && p.w1)) {
+      block_sum2_256(sa, sb, red);
+      if (p.w0) ra = 1.0f / sqrtf(sa * inv_n + p.eps);
+      if (b && p.w1) rb = 1.0f / sqrtf(sb * inv_n + p.eps);
+    }
+    auto joined = [&](float ya, float yb, float wa, float wb) {
+      float s = p.w0 ? ya * ra * wa : ya;
+      if (b) s += p.w1 ? yb * rb * wb : yb;
       return s * p.coef;
+    };
+    auto joined_at = [&](int i) {
+      return joined(a[i], b ? b[i] : 0.0f, p.w0 ? p.w0[i] : 1.0f, (b && p.w1) ? p.w1[i] : 1.0f);
     };
     float ss = 0.0f;
 #pragma unroll
     for (int e = 0; e < CPT; ++e) {
-      const int i = tid + 256 * e;
-      av[e] = i < n ? joined(i, av[e], bv[e]) : 0.0f;  // (av now holds the joined value)
+      av[e] = tid + 256 * e < n ? joined(av[e], bv[e], w0[e], w1[e]) : 0.0f;  // (av now holds the joined value)
       ss = fmaf(av[e], av[e], ss);
     }
     for (int i = tid + 256 * CPT; i < n; i += 256) {
-      const float s = joined(i, a[i], b ? b[i] : 0.0f);
+      const float s = joined_at(i);
       ss = fmaf(s, s, ss);
     }
     const float rs = 1.0f / sqrtf(block_sum_256(ss, red) * inv_n + p.eps);
@@ -252,11 +279,11 @@ __global__ void __launch_bounds__(256) sandwich_step_kernel(SandwichArgs p) {
     for (int e = 0; e < CPT; ++e) {
       const int i = tid + 256 * e;
       if (i < n) {
-        xv[e] = fmaf(av[e] * rs, p.post_w[i], xv[e]);
+        xv[e] = fmaf(av[e] * rs, wp[e], xv[e]);
         xr[i] = xv[e];
       }
     }
-    for (int i = tid + 256 * CPT; i < n; i += 256) xr[i] = fmaf(joined(i, a[i], b ? b[i] : 0.0f) * rs, p.post_w[i], xr[i]);
+    for (int i = tid + 256 * CPT; i < n; i += 256) xr[i] = fmaf(joined_at(i) * rs, p.post_w[i], xr[i]);
   }
   if (!p.next_w) return;
   float sx = 0.0f;
@@ -264,15 +291,20 @@ __global__ void __launch_bounds__(256) sandwich_step_kernel(SandwichArgs p) {
   for (int e = 0; e < CPT; ++e) sx = fmaf(xv[e], xv[e], sx);
   for (int i = tid + 256 * CPT; i < n; i += 256) sx = fmaf(xr[i], xr[i], sx);  // (written by this thread above)
   const float rx = 1.0f / sqrtf(block_sum_256(sx, red) * inv_n + p.eps);
-  auto put = [&](int i, float v) {
-    const float o = v * rx * p.next_w[i];
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) {
+    const int i = tid + 256 * e;
+    if (i < n) {
+      const float o = xv[e] * rx * wn[e];
+      if (p.h) p.h[r * n + i] = o;
+      if (p.h16) p.h16[r * n + i] = f2bf(o);
+    }
+  }
+  for (int i = tid + 256 * CPT; i < n; i += 256) {
+    const float o = xr[i] * rx * p.next_w[i];
     if (p.h) p.h[r * n + i] = o;
     if (p.h16) p.h16[r * n + i] = f2bf(o);
-  };
-#pragma unroll
-  for (int e = 0; e < CPT; ++e)
-    if (tid + 256 * e < n) put(tid + 256 * e, xv[e]);
-  for (int i = tid + 256 * CPT; i < n; i += 256) put(i, xr[i]);
+  }
 }
 
 }  // namespace lgs

@@ -669,20 +669,25 @@ def test_checkpoint_folder_through_registry_and_runner(tmp_path):
     from lit_gpt.layered import LayeredGPT
 
     REPO = Path(__file__).resolve().parent.parent
-    cfg = make_cfg(MIXED)
-    weights = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=11)
-    (tmp_path / "config.json").write_text(json.dumps(cfg))
-    save_file({k: v.contiguous() for k, v in weights.items()}, str(tmp_path / "model.safetensors"))
-    config = load_config(tmp_path)
-    assert model_class(config) is LayeredGPT
-    a, b = tokens_of(14, cfg["vocab"], seed=1), tokens_of(6, cfg["vocab"], seed=2)
-    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:10], "want": [3, 9]}, {"id": "b", "tokens": b[:5], "want": []}], "end": []},
-             {"step": 1, "entries": [{"id": "a", "tokens": a[10:11], "want": [0]}, {"id": "b", "tokens": b[5:], "want": [0]}], "end": ["b"]},
-             {"step": 2, "entries": [{"id": "a", "tokens": a[11:12], "want": []}], "end": []},
-             {"step": 3, "entries": [{"id": "a", "tokens": a[12:], "want": [1]}], "end": ["a"]}]
-    out = tmp_path / "out"
-    for dtype, tol in (("float32", TOL32), ("bfloat16", TOL16)):
-        r = subprocess.run([sys.executable, str(REPO / "bin" / "trace_run"), "--model", str(tmp_path), "--dtype", dtype,
+    # (bf16 on layers without routing: a near tie of a router may flip under bf16 products, and what a flipped token
+    # leaves in the caches and states moves every later row)
+    plain = [(key_pair(), dense()), (rope_pair(scaling=SCALING), dense(ff=20)), (key_pair(heads=3, kv_heads=3, dim=6, every=0, rheads=2), None)]
+    for dtype, tol, layers in (("float32", TOL32, MIXED), ("bfloat16", TOL16, plain)):
+        cfg = make_cfg(layers)
+        weights = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=11)
+        folder = tmp_path / dtype
+        folder.mkdir()
+        (folder / "config.json").write_text(json.dumps(cfg))
+        save_file({k: v.contiguous() for k, v in weights.items()}, str(folder / "model.safetensors"))
+        config = load_config(folder)
+        assert model_class(config) is LayeredGPT
+        a, b = tokens_of(14, cfg["vocab"], seed=1), tokens_of(6, cfg["vocab"], seed=2)
+        steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:10], "want": [3, 9]}, {"id": "b", "tokens": b[:5], "want": []}], "end": []},
+                 {"step": 1, "entries": [{"id": "a", "tokens": a[10:11], "want": [0]}, {"id": "b", "tokens": b[5:], "want": [0]}], "end": ["b"]},
+                 {"step": 2, "entries": [{"id": "a", "tokens": a[11:12], "want": []}], "end": []},
+                 {"step": 3, "entries": [{"id": "a", "tokens": a[12:], "want": [1]}], "end": ["a"]}]
+        out = folder / "out"
+        r = subprocess.run([sys.executable, str(REPO / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype,
                             "--out", str(out), "--max-tokens", "32"], input="\n".join(json.dumps(s) for s in steps) + "\n",
                            capture_output=True, text=True, timeout=300)
         assert r.returncode == 0, r.stderr[-2000:]
@@ -692,6 +697,6 @@ def test_checkpoint_folder_through_registry_and_runner(tmp_path):
         got1 = torch.from_numpy(np.fromfile(out / "1.f32", dtype="<f4").reshape(2, -1))
         got3 = torch.from_numpy(np.fromfile(out / "3.f32", dtype="<f4").reshape(1, -1))
         assert not (out / "2.f32").exists()
-        err = torch.cat([rel_err(got0, la[[3, 9]]), rel_err(got1, torch.stack([la[10], lb[5]])), rel_err(got3, la[13:14])])
-        # (bf16: a near tie of the router may flip and move a row, so the bulk of the rows is what is compared)
-        assert (err.max() if dtype == "float32" else err.median()) < tol
+        assert rel_err(got0, la[[3, 9]]).max() < tol
+        assert rel_err(got1, torch.stack([la[10], lb[5]])).max() < tol
+        assert rel_err(got3, la[13:14]).max() < tol
