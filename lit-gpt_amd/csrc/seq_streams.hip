@@ -202,7 +202,7 @@ struct SandwichArgs {
   int n;
 };
 
-// sums of two values over the 256 threads of a workgroup in one round (`red` holds 8 floats)
+// sums of two values over the 256 threads of a workgroup at once (`red` holds 8 floats)
 __device__ __forceinline__ void block_sum2_256(float& u, float& v, float* red) {
   u = wave_sum(u);
   v = wave_sum(v);
@@ -224,7 +224,7 @@ __global__ void __launch_bounds__(256) sandwich_step_kernel(SandwichArgs p) {
   float* xr = p.x + r * n;
   const float inv_n = 1.0f / (float)n;
   // every operand of the registers' share of the row is fetched up front, so that the reductions below wait for
-  // one round of loads only
+  // one batch of loads only
   float xv[CPT], av[CPT], bv[CPT], w0[CPT], w1[CPT], wp[CPT], wn[CPT];
   const float *a = p.y0 ? p.y0 + r * n : nullptr, *b = p.y1 ? p.y1 + r * n : nullptr;
 #pragma unroll
