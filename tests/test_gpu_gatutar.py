@@ -672,8 +672,8 @@ def test_checkpoint_folder_through_registry_and_runner(tmp_path):
     # (bf16 on layers without routing: a near tie of a router may flip under bf16 products, and what a flipped token
     # leaves in the caches and states moves every later row)
     plain = [(key_pair(), dense()), (rope_pair(scaling=SCALING), dense(ff=20)), (key_pair(heads=3, kv_heads=3, dim=6, every=0, rheads=2), None)]
-    for dtype, tol, layers in (("float32", TOL32, MIXED), ("bfloat16", TOL16, plain)):
-        cfg = make_cfg(layers)
+    for dtype, tol, layers, width in (("float32", TOL32, MIXED, 40), ("bfloat16", TOL16, plain, 136)):
+        cfg = make_cfg(layers, width=width)
         weights = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=11)
         folder = tmp_path / dtype
         folder.mkdir()
