@@ -643,6 +643,23 @@ def test_captured_decode_step_replays():
     assert outs == eager
 
 
+def test_command_line_serves_a_checkpoint_folder(tmp_path, capsys):
+    from safetensors.torch import save_file
+
+    from generate.base import main
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+
+    cfg = make_cfg(MIXED[:3], vocab=70)
+    w = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=15)
+    save_file({k: v.contiguous() for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    main(checkpoint_dir=tmp_path, max_new_tokens=5, temperature=0.0, top_k=None, prompt_len=7, precision="32-true")
+    ids = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert len(ids) == 12
+    assert follows_plain_greedy(cfg, w, ids[:7], ids)
+
+
 def test_two_streams_against_one():
     from lit_gpt.mixers import ParallelMixer
 
