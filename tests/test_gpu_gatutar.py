@@ -272,6 +272,24 @@ def test_batch_of_unequal_requests_against_each_alone(mixed):
     assert not eng.live
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_many_sequences_decoded_together(dtype):
+    """More than eight one-token rows in a step (the matrix-core products' row count, the second stream) against
+    each request alone; layers without routing, so that bf16 holds no hard choices."""
+    layers = [(key_pair(), dense()), (rope_pair(scaling=SCALING), dense(ff=20)), (key_pair(heads=3, kv_heads=3, dim=6, every=0, rheads=2), None)]
+    cfg = make_cfg(layers, width=72)
+    model, _ = build(cfg, dtype=dtype, seed=13)
+    seqs = [tokens_of(5 + 3 * i, cfg["vocab"], seed=200 + i) for i in range(12)]
+    alone = [engine_logits(model, [s], [[len(s) - 4] + [1] * 4])[0] for s in seqs]
+    from generate.batch import BatchEngine
+
+    eng = BatchEngine(model, max_seq_length=48, slots=3)
+    together = engine_logits(model, seqs, [[len(s) - 4] + [1] * 4 for s in seqs], engine=eng)
+    tol = SAME if dtype == torch.float32 else TOL16
+    for a, b in zip(together, alone):
+        assert rel_err(a, b).max() < tol
+
+
 def test_slots_freed_and_used_again(mixed):
     cfg, model, _ = mixed
     from generate.batch import BatchEngine
