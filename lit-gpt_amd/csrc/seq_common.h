@@ -1,6 +1,6 @@
-// Shared declarations of liblitgpt_seq.so: the kernels of the layered models (retention, latent-, differential- and
-// sink-attention, state-space and delta-rule mixers, gated feed-forwards, sparse experts, per-layer token inputs) over
-// an fp32 residual stream.
+// Shared declarations of liblitgpt_seq.so: the kernels of the layered models (retention, latent-, differential-,
+// sink- and rotary attention, state-space, delta-rule and gated linear-attention mixers, gated and ungated
+// feed-forwards, sparse experts, per-layer token inputs) over an fp32 residual stream.
 //
 // Conventions: activations are fp32 in memory in both precisions. A weight matrix is [out][in], either bf16 (raw
 // uint16; the activation operand of a product is then rounded to bf16 and the sum is fp32: the matrix-core

@@ -3,9 +3,13 @@
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 // g is one number per head, or one per head and key channel (the rows of S). Query / key heads may be shared by
 // groups of value heads (head h reads q / k head h / (H / G)). Everything that enters the recurrence is fp32.
+// The same kernels serve the plain gated rule without the correction, S <- diag(g) S + k v^T (gated linear attention:
+// u = v, no beta), whose decay is sigmoid(raw + bias)^(1 / tau) and whose q is only scaled.
 //
-//   lgs_delta_prepare   per token: q and k (after their convolution) become unit vectors per head, q times q_scale;
-//                       beta = sigmoid(raw); g = exp(-exp(A_log) softplus(raw + dt_bias)); k . q per key head
+//   lgs_delta_prepare   per token: q and k (after their convolution) become unit vectors per head, q times q_scale
+//                       (or q is only scaled); beta = sigmoid(raw); g = exp(-exp(A_log) softplus(raw + dt_bias)) or
+//                       sigmoid(raw + bias)^(1 / tau); k . q per key head. Steps of few rows spread the decays (each
+//                       a low-rank product) over workgroups of their own
 //   lgs_delta_step_prepare  the same for a step in which every sequence brings one token, with the short convolution
 //                       of q | k | v (and the shift of its stored inputs) in the same launch
 //   lgs_gated_delta     the recurrence, token by token for every step kind. The columns of S never mix, so a column

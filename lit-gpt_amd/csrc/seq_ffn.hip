@@ -4,8 +4,11 @@
 //   lgs_glu_clamped      out = g sigmoid(alpha g) (u + shift) with g = min(a, limit), u = clamp(b, -limit, limit)
 //   lgs_moe_route        per token: the `top` largest router logits (fp32, lowest index first among equals) and the
 //                        softmax over just those
-//   lgs_moe_route_scores per token: softmax over all router outputs; the choice adds a stored correction to the
-//                        scores, the weights are the chosen scores themselves
+//   lgs_moe_route_scores per token: softmax over all router outputs (or the sigmoid of each on its own); the choice
+//                        adds a stored correction to the scores, the weights are the chosen scores themselves (or
+//                        their squares: a score on the input of an expert with a relu^2 activation)
+//   lgs_act_rows         out = act(a) times an optional sigmoid gate of one number per row (an ungated unit whose
+//                        up-projection is part of a fused product: the shared expert)
 //   lgs_moe_up / _down   the routed experts as streaming GEMVs over (token, choice) pairs: only the chosen experts'
 //                        rows are read; the down kernel sums a token's choices in their routing order and adds the
 //                        result to the residual stream (the decode form; a prompt runs grouped products instead)

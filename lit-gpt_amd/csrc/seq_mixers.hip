@@ -1,7 +1,8 @@
 // Sequence mixers of the layered models, all sums in fp32.
 //
-//   lgs_retention        decayed linear attention: rotary (half layout) on q and k, k scaled, then per head
-//                        S <- decay S + k v^T, o = S^T q, the state S (d x dv fp32) carried per cache slot
+//   lgs_retention        decayed linear attention: an optional activation on q, k and v, rotary (half layout) on q
+//                        and k, k scaled, then per head S <- decay S + k v^T, o = S^T q, the state S (d x dv fp32)
+//                        carried per cache slot
 //   lgs_head_gate        per head: optional unit RMS of o, times act(g): the retention's output norm + silu gate and
 //                        the latent attention's sigmoid gate
 //   lgs_latent_prepare   latent attention, per token: RMS-normed latent c and the rotated shared key part go to the

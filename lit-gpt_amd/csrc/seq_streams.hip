@@ -7,6 +7,9 @@
 //   lgs_embed_streams   x[t][j] = table[tokens[t]] * scale for every stream j
 //   lgs_streams_step    one launch per sublayer boundary: the write-back of the sublayer that just ran (optional)
 //                       followed by the read + norm of the next one (optional), so the streams are read once
+//   lgs_sandwich_step   the boundary of layers whose sublayers are normed on the way in and out (one stream): the
+//                       norms and the average of up to two branch outputs, the output norm times the layer scale,
+//                       the residual add and the next sublayer's input norm in one launch
 #include "seq_common.h"
 
 namespace lgs {

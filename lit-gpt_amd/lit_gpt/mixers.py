@@ -6,9 +6,11 @@ gate and up matrices, the router), and each module finds its columns in the resu
 module's rows of that matrix, ``bind`` tells it where they landed. Outputs are accumulated into the fp32 residual
 stream ``x`` by the epilogue of the out-projection (or the expert combine), so a layer needs no add kernel.
 
-Mixers here: ``Retention``, ``LatentAttention``, ``DiffAttention``, ``SelectiveScan``, ``GatedDelta`` (the gated delta
-rule with a decay per head or per head and key channel), ``SinkAttention`` (unit-RMS queries and keys, a query
-temperature, a sink in the normaliser) and ``ParallelMixer`` (the last two side by side on one input projection).
+Mixers here: ``Retention`` (and its preset ``Lightning``: the constant-decay rule on activated projections),
+``LatentAttention``, ``DiffAttention``, ``SelectiveScan``, ``GatedDelta`` (the gated delta rule with a decay per head or
+per head and key channel), ``GatedLinearAttention`` (the gated rule without the correction), ``SinkAttention`` (one-map
+softmax attention: optional q / k norms, rotary positions, a query temperature, a learned or constant sink, values that
+are the keys, a gate per head) and ``ParallelMixer`` (two of them side by side on one input projection).
 
 A step is a packed batch (``StepBatch``): the tokens of all sequences row after row, with per-token cache slot and
 position and per-sequence row range, slot and first position, all int32 on the device. Sizes, decays, scales, rotary
