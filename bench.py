@@ -750,8 +750,8 @@ def sandwich_bench(args) -> None:
                       "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(1, H // 2 - 1)) for i in range(H // 2)]}}}
         rot = {"type": "parallel", "mixer": {
             "left": {"heads": H, "kv_heads": H // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                     "rot": {"dims": 64, "base": 5e5, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
-            "right": {"heads": H // 2, "dim": 128, "vdim": 128, "tau": 16.0, "decay_rank": W // 32}}}
+                     "rot": {"dims": 64, "base": 5e5, "scaling": {"factor": 4.0, "low": 1.0, "high": 2.0, "original": 4096}}},
+            "right": {"heads": H // 2, "dim": 128, "vdim": 128, "tau": 8.0, "decay_rank": W // 32}}}
         cfg = LayeredConfig.from_dict({"architecture": "Gatutar", "vocab": V, "width": W, "norm": {"eps": 1e-5},
                                        "layers": [dict(kv, mlp=dense), dict(rot, mlp=moe), dict(kv, mlp=dense),
                                                   dict(rot, mlp=moe)]})
